@@ -6,3 +6,4 @@ from .registry import (  # noqa: F401
 from .llama import LlamaConfig  # noqa: F401
 from .mamenex import MamenexConfig  # noqa: F401
 from .nagezen import NagezenConfig  # noqa: F401
+from .milenex import MilenexConfig  # noqa: F401

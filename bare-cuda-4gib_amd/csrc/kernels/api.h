@@ -309,6 +309,9 @@ struct bc4g_prepare_section {
   long in_row, out_row, page_stride, head_stride, token_stride;
   int in_dtype, out_dtype, half, page_tokens, heads, dim;
   float eps, factor;
+  // pairing 0: element i turns with element i + half, 1: element 2i with element 2i + 1.  unit_after 1: after the
+  // rotation the head is divided by sqrt(mean(head^2) + eps), without a weight.
+  int pairing, unit_after;
 };
 int bc4g_heads_prepare_many(const bc4g_prepare_section* sections, int n_sections, int n_rows, void* stream);
 int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, const float* bias, const float* norm_w, float eps,
@@ -334,10 +337,45 @@ int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_scale, const
 // [T, heads, maps, dim]; keys [page, kv_head * maps + map, token, dim], values [page, kv_head, token, vdim]; a row at p
 // sees j <= p with p - j < window or j < keep_first (window 0: all).  o = a1 - lambda a2 (one map: a1), with normalize
 // divided by sqrt(mean(o^2) + eps), times factor, times act(gate) (1: silu, 2: sigmoid; gate null: none).  waves (1 to 8):
-// how many waves cut one row's keys among them.
+// how many waves cut one row's keys among them.  sink [heads] (or null): exp(sink) joins every map's denominator.
+// far1, far2 [heads] (both or neither): far1 ln(1 + far2 (p - j)) is taken off the scaled score.
 int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
                         const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                         float lambda, int normalize, float eps, float factor, const void* gate, int gate_dtype, long gate_row,
                         int gate_act, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
-                        int vdim, int page_tokens, int window, int keep_first, float scale, int waves, void* stream);
+                        int vdim, int page_tokens, int window, int keep_first, float scale, int waves, const float* sink,
+                        const float* far1, const float* far2, void* stream);
+
+// Windowed softmax attention whose heads' weights are mixed before they meet the values (attention_talk.hip): q float32
+// [T, heads, dim]; keys [page, kv_head, token, dim], values [page, kv_head, token, vdim]; a row at p sees j <= p with
+// p - j < window (0: all).  score = q . k * scale - far1 ln(1 + far2 (p - j)); w_g = exp(score_g) / (sum_j exp(score_g)
+// + exp(sink_g)); head h weighs the values of its own key/value head by sum_g talk[h, g] w_g; times sigmoid(gate[t, h])
+// if a gate [T, heads] is given (rows gate_row apart).  sink, far1/far2 and talk ([heads, heads]) may each be null.
+// heads * dim at most 8192, heads at most 64.
+int bc4g_attention_talk(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
+                        const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
+                        const float* sink, const float* far1, const float* far2, const float* talk, const void* gate,
+                        int gate_dtype, long gate_row, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads,
+                        int dim, int vdim, int page_tokens, int window, float scale, void* stream);
+
+// out[t, :] += float(table[ids[t], :]): the embedding once more, added to the stream.
+int bc4g_embed_add(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden, int vocab,
+                   void* stream);
+
+// z -> z Phi(z) (the exact gelu, by erf), element by element; out may be the input.
+int bc4g_gelu(const void* in, void* out, int dtype, long total, void* stream);
+
+// The choice of experts for every row (moe.hip).  logits float32 [T, >= experts] (rows logits_row apart): s =
+// softmax over the experts; choice = s + correction (null: s); the experts lie in `groups` equal groups of neighbours, a
+// group counts by its largest choice, and only experts of the `keep` best groups can be chosen; the `top` largest
+// choices win (the lower index among equals).  weights float32 [T, experts]: s of the chosen, 0 elsewhere.
+// chosen int32 [T, top] (may be null).  experts at most 1024.
+int bc4g_moe_route(const float* logits, long logits_row, const float* correction, float* weights, int32_t* chosen,
+                   int n_rows, int experts, int groups, int keep, int top, void* stream);
+// Clamped gated units of all experts side by side, weighted: gu [T, experts * 2 ff + 2 shared_ff] holds per expert its
+// ff gates, then its ff ups, and last the shared unit's gates and ups; out [T, experts * ff + shared_ff] =
+// weights[t, e] * g sigmoid(slope g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), the shared unit
+// (its own limit) weighted by sigmoid(shared_logit[t]) (float32, rows shared_row apart; null with shared_ff 0).
+int bc4g_routed_glu(const void* gu, void* out, int dtype, const float* weights, const float* shared_logit, long shared_row,
+                    float limit, float shared_limit, float slope, int n_rows, int experts, int ff, int shared_ff, void* stream);
 }

@@ -1,7 +1,9 @@
 // Softmax attention over a paged cache whose query heads carry one or two score maps over the same values
 // (differential attention: o = a1 - lambda a2), with a window of the last keys plus the first few keys of the
 // sequence, keys and values of different sizes, and the head's output optionally divided by its root mean square,
-// scaled and gated.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
+// scaled and gated.  Two further options, each a vector with one number a query head: a sink -- exp(sink) joins the
+// softmax's denominator, with no key and no value, never scaled -- and a penalty on distance, r1 ln(1 + r2 (p - j)),
+// taken off the scaled score.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
 //
 // A row at position p sees key j if j <= p and (window == 0 or p - j < window or j < keep_first); kept keys keep their
 // own positions (they were rotated when they were written).  One workgroup per (row, query head): the visible keys --
@@ -60,7 +62,8 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ positions, float lambda, int normalize, float eps, float factor,
     const void* __restrict__ gate, int gate_dtype, long gate_row, int gate_act, void* __restrict__ out, int out_dtype,
-    int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens, int window, int keep_first, float scale) {
+    int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens, int window, int keep_first, float scale,
+    const float* __restrict__ sink, const float* __restrict__ far1, const float* __restrict__ far2) {
   __shared__ __align__(16) float q_s[MAPS][kMaxDim];
   __shared__ float p_s[kNW][MAPS][kWave];
   __shared__ long v_at[kNW][kWave];           // where every key of the wave's tile has its values
@@ -81,6 +84,7 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int kept = window > 0 ? (keep_first < first ? keep_first : first) : 0;      // kept keys before the window
   const int total = kept + (pos - first + 1);
+  const float pen1 = far1 ? far1[head] : 0.f, pen2 = far1 ? far2[head] : 0.f;
   const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
   constexpr int VPL = 4;                // value dimensions a lane holds
   constexpr int KPI = LPK ? kWave / LPK : 1;      // keys a load of values brings
@@ -154,7 +158,9 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
         const T* kp = k_cache + ((page * (n_kv_heads * MAPS) + kvh * MAPS + m) * page_tokens + off) * dim;
         for (int c = 0; c < dim; ++c) dot = fmaf(q_s[m][c], to_float(kp[c]), dot);
       }
-      const float sc = seen ? dot * scale : -INFINITY;
+      float sc = dot * scale;
+      if (far1) sc -= pen1 * log1pf(pen2 * static_cast<float>(pos - j));
+      if (!seen) sc = -INFINITY;
       const float m_new = fmaxf(mx[m], wave_max(sc));       // finite: the tile's first key is visible
       const float p = seen ? expf(sc - m_new) : 0.f;
       const float alpha = expf(mx[m] - m_new);               // 0 on the wave's first tile
@@ -225,6 +231,17 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
 #pragma unroll
         for (int i = 0; i < VPL; ++i) acc[m][i] = fmaf(part_acc[w][m][vcol[i]], f, acc[m][i]);
       }
+      mx[m] = top;                                       // (what the merged sums are counted from)
+    }
+  }
+  if (sink) {                                            // the sink: a term of the denominator, with no value
+    const float sk = sink[head];
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) {
+      const float top = fmaxf(mx[m], sk), f = expf(mx[m] - top);
+      sum[m] = fmaf(sum[m], f, expf(sk - top));
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) acc[m][i] *= f;
     }
   }
   float o[VPL];
@@ -259,7 +276,8 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
                                    const int32_t* positions, float lambda, int normalize, float eps, float factor,
                                    const void* gate, int gate_dtype, long gate_row, int gate_act, void* out, int out_dtype,
                                    int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int page_tokens,
-                                   int window, int keep_first, float scale, int waves, void* stream) {
+                                   int window, int keep_first, float scale, int waves, const float* sink,
+                                   const float* far1, const float* far2, void* stream) {
   BC4G_REQUIRE(waves >= 1 && waves <= kMaxWaves, "attention_maps: %d waves a row (1 to %d)", waves, kMaxWaves);
   BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= 65535 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "attention_maps: bad sizes T=%d heads=%d/%d", n_rows, n_heads, n_kv_heads);
@@ -273,6 +291,7 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
                (gate_act == 1 || gate_act == 2 || !gate) && (out_dtype == kF32 || out_dtype == kBF16) &&
                (!gate || gate_dtype == kF32 || gate_dtype == kBF16),
                "attention_maps: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
+  BC4G_REQUIRE((far1 == nullptr) == (far2 == nullptr), "attention_maps: the distance penalty needs both of its vectors");
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_rows, n_heads);
@@ -287,7 +306,7 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
   attention_maps_kernel<T, M, W, V, E><<<grid, waves * kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
                                                      block_table, table_stride, row_seq, positions, lambda, normalize, eps, \
                                                      factor, gate, gate_dtype, gate_row, gate_act, out, out_dtype, n_heads,  \
-                                                     n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale)
+                                                     n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale, sink, far1, far2)
   if (cache_dtype == kF32) {
     if (maps == 1) BC4G_MAPS(float, 1); else BC4G_MAPS(float, 2);
   } else if (cache_dtype == kBF16) {

@@ -1,0 +1,312 @@
+// Windowed softmax attention over a paged cache whose heads' weights are mixed by a matrix before they meet the values
+// ("talking heads" after the softmax), with a sink in every head's denominator, a penalty on distance in the scores and
+// a gate per head on the output.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
+//
+//   score_g(p, j) = q_g . k_j * scale - far1_g ln(1 + far2_g (p - j))            for p - window < j <= p
+//   w_g(p, j)     = exp(score_g) / (sum over the visible j of exp(score_g) + exp(sink_g))
+//   o_h(p)        = sigmoid(gate_h(p)) * sum_j (sum_g talk[h, g] w_g(p, j)) v_j       with the values of h's own key/value head
+//
+// The mixing needs every head's finished weight at a key, and a weight is finished only when its row's denominator is
+// known: so a workgroup is one row with all its heads, and it walks the row's keys twice.  The first walk leaves every
+// head's maximum and denominator; the second works the scores out again, turns them into weights in LDS (head x 64 keys),
+// mixes them and adds the values up.  A wave owns the heads w, w + waves, ...: their scores, their statistics, their
+// outputs.  Against keeping the scores of the first walk (heads x window floats a row) the second product costs less than
+// the memory would.  Caches: keys [page, kv_head, token, dim], values [page, kv_head, token, vdim].
+#include <float.h>
+#include <math.h>
+
+#include "api.h"
+#include "common.h"
+
+namespace bc4g {
+namespace {
+
+constexpr int kMaxWaves = 8;
+constexpr int kMaxHeads = 64;
+constexpr int kMaxDim = 256, kMaxVdim = 256;
+constexpr int kMaxQ = 8192;      // heads * (dim rounded up to 32): what the queries may take in LDS
+constexpr int kAhead = 8;        // keys whose values a lane asks for together
+
+__device__ inline float4 load_four(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ inline float4 load_four(const bf16_t* p) {
+  const uint2 bits = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(bits.x << 16), __uint_as_float(bits.x & 0xffff0000u),
+                     __uint_as_float(bits.y << 16), __uint_as_float(bits.y & 0xffff0000u));
+}
+
+__device__ inline void wave_sync() {      // LDS written by this wave's lanes is read by its other lanes
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// SL: heads a wave owns at most.  E4: for the scores eight lanes share a key, each with 4 E4 of its dimensions
+// (dim <= 32 E4).  LPK: lanes that share a key for the weighted sums, each with four neighbouring value dimensions
+// (vdim <= 4 LPK); 0: a lane holds dimensions lane, lane + 64, ... (any vdim).
+template <typename T, int SL, int E4, int LPK>
+__global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
+    const float* __restrict__ q, long q_row, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ positions, const float* __restrict__ sink, const float* __restrict__ far1,
+    const float* __restrict__ far2, const float* __restrict__ talk, const void* __restrict__ gate, int gate_dtype,
+    long gate_row, void* __restrict__ out, int out_dtype, int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens,
+    int window, float scale) {
+  extern __shared__ __align__(16) float dyn[];
+  __shared__ long k_at[kMaxWaves][kWave];     // where every key of the tile lies (key/value head 0)
+  __shared__ long v_at[kMaxWaves][kWave];
+  __shared__ float s_s[kMaxWaves][kWave];     // a head's scores on their way from (key, piece) lanes to lane = key
+  __shared__ float m_s[kMaxWaves][kWave];     // a head's mixed weights, lane = key -> every lane
+  const int dimp = 32 * E4;                   // a head's queries in LDS, zeros beyond dim
+  float* q_s = dyn;                           // [heads][dimp]
+  float* p_s = dyn + n_heads * dimp;          // [heads][64]: the tile's weights
+  const int row = blockIdx.x, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int n_waves = blockDim.x / kWave;
+  const int per_kv = n_heads / n_kv_heads;
+  const int pos = positions[row];
+  const int32_t* table = block_table + static_cast<long>(row_seq[row]) * table_stride;
+  for (int i = threadIdx.x; i < n_heads * dimp; i += blockDim.x) {
+    const int h = i / dimp, c = i % dimp;
+    q_s[i] = c < dim ? q[row * q_row + static_cast<long>(h) * dim + c] : 0.f;
+  }
+  __syncthreads();
+
+  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int total = pos - first + 1;
+  const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
+  const int sub = lane / 8, piece = lane % 8;
+  int k_col[E4];
+#pragma unroll
+  for (int e = 0; e < E4; ++e) {
+    const int c = piece * 4 * E4 + 4 * e;
+    k_col[e] = c + 4 <= dim ? c : (dim >= 4 ? dim - 4 : 0);
+  }
+  const long k_head = static_cast<long>(page_tokens) * dim, v_head = static_cast<long>(page_tokens) * vdim;
+
+  // The scores of head h for the wave's tile (k_at filled, synchronized): lane = key.  Lanes without a key compute on
+  // the tile's first key; the caller drops them.
+  auto scores = [&](int h, int j) -> float {
+    const int kvh = h / per_kv;
+    float dot;
+    if (by_four) {
+      float4 q_r[E4];
+#pragma unroll
+      for (int e = 0; e < E4; ++e) q_r[e] = *reinterpret_cast<const float4*>(&q_s[h * dimp + piece * 4 * E4 + 4 * e]);
+#pragma unroll
+      for (int it = 0; it < 8; it += 2) {                  // sixteen keys' pieces asked for together
+        float4 kk[2][E4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const T* kp = k_cache + k_at[wave][8 * (it + u) + sub] + kvh * k_head;
+#pragma unroll
+          for (int e = 0; e < E4; ++e) kk[u][e] = load_four(kp + k_col[e]);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          float part = 0.f;
+#pragma unroll
+          for (int e = 0; e < E4; ++e) {
+            part = fmaf(q_r[e].x, kk[u][e].x, part), part = fmaf(q_r[e].y, kk[u][e].y, part);
+            part = fmaf(q_r[e].z, kk[u][e].z, part), part = fmaf(q_r[e].w, kk[u][e].w, part);
+          }
+          part += __shfl_xor(part, 1, kWave), part += __shfl_xor(part, 2, kWave), part += __shfl_xor(part, 4, kWave);
+          if (piece == 0) s_s[wave][8 * (it + u) + sub] = part;
+        }
+      }
+      wave_sync();
+      dot = s_s[wave][lane];
+      wave_sync();
+    } else {
+      const T* kp = k_cache + k_at[wave][lane] + kvh * k_head;
+      dot = 0.f;
+      for (int c = 0; c < dim; ++c) dot = fmaf(q_s[h * dimp + c], to_float(kp[c]), dot);
+    }
+    float sc = dot * scale;
+    if (far1) sc -= far1[h] * log1pf(far2[h] * static_cast<float>(pos - j));
+    return sc;
+  };
+  auto place = [&](int v0, bool& seen, int& j) {      // this lane's key of the tile that begins at visible key v0
+    seen = v0 + lane < total;
+    j = first + (seen ? v0 + lane : v0);
+    const long page = table[j / page_tokens];
+    const int off = j % page_tokens;
+    k_at[wave][lane] = (page * n_kv_heads * page_tokens + off) * dim;
+    v_at[wave][lane] = (page * n_kv_heads * page_tokens + off) * vdim;
+    wave_sync();
+  };
+
+  // ---- first walk: every head's maximum and denominator --------------------------------------------------------------
+  float mx[SL], inv[SL];
+#pragma unroll
+  for (int s = 0; s < SL; ++s) mx[s] = -INFINITY, inv[s] = 0.f;
+  for (int v0 = 0; v0 < total; v0 += kWave) {
+    bool seen;
+    int j;
+    place(v0, seen, j);
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const int h = wave + s * n_waves;
+      if (h >= n_heads) break;
+      float sc = scores(h, j);
+      if (!seen) sc = -INFINITY;
+      const float m_new = fmaxf(mx[s], wave_max(sc));       // finite: the tile's first key is visible
+      const float p = seen ? expf(sc - m_new) : 0.f;
+      inv[s] = inv[s] * expf(mx[s] - m_new) + wave_sum(p);  // (the sum so far; turned into its inverse below)
+      mx[s] = m_new;
+    }
+    wave_sync();
+  }
+#pragma unroll
+  for (int s = 0; s < SL; ++s) {
+    const int h = wave + s * n_waves;
+    if (h >= n_heads) break;
+    float sum = inv[s];
+    if (sink) {                                            // the sink: a term of the denominator, never scaled
+      const float sk = sink[h], top = fmaxf(mx[s], sk);
+      sum = fmaf(sum, expf(mx[s] - top), expf(sk - top));
+      mx[s] = top;
+    }
+    inv[s] = 1.0f / sum;
+  }
+
+  // ---- second walk: weights, mixed, times values ------------------------------------------------------------------------
+  constexpr int VPL = 4;
+  constexpr int KPI = LPK ? kWave / LPK : 1;      // keys a load of values brings
+  const int vgroup = LPK ? lane / LPK : 0;
+  int vcol[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) vcol[i] = LPK ? 4 * (lane % (LPK ? LPK : 1)) + i : lane + i * kWave;
+  const int vfrom = LPK ? (vcol[0] + 4 <= vdim ? vcol[0] : vdim - 4) : 0;
+  float acc[SL][VPL];
+#pragma unroll
+  for (int s = 0; s < SL; ++s)
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) acc[s][i] = 0.f;
+  for (int v0 = 0; v0 < total; v0 += kWave) {
+    bool seen;
+    int j;
+    place(v0, seen, j);
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const int h = wave + s * n_waves;
+      if (h >= n_heads) break;
+      const float sc = scores(h, j);
+      p_s[h * kWave + lane] = seen ? expf(sc - mx[s]) * inv[s] : 0.f;
+    }
+    __syncthreads();                                        // every head's weights of this tile are there
+    const int n_here = total - v0 < kWave ? total - v0 : kWave;
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const int h = wave + s * n_waves;
+      if (h >= n_heads) break;
+      float mixed;
+      if (talk) {
+        mixed = 0.f;
+        for (int g = 0; g < n_heads; ++g) mixed = fmaf(talk[h * n_heads + g], p_s[g * kWave + lane], mixed);
+      } else {
+        mixed = p_s[h * kWave + lane];
+      }
+      m_s[wave][lane] = mixed;
+      wave_sync();
+      const long v_off = (h / per_kv) * v_head;
+      for (int j0 = 0; j0 < n_here; j0 += kAhead * KPI) {  // (keys beyond the tile's last weigh zero and read the first key's values)
+        float vv[kAhead][VPL];
+#pragma unroll
+        for (int b = 0; b < kAhead; ++b) {
+          const T* vrow = v_cache + v_at[wave][(j0 + b * KPI + vgroup) % kWave] + v_off;
+          if (LPK) {
+            const float4 four = load_four(vrow + vfrom);
+            vv[b][0] = four.x, vv[b][1] = four.y, vv[b][2] = four.z, vv[b][3] = four.w;
+          } else {
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) vv[b][i] = to_float(vrow[vcol[i] < vdim ? vcol[i] : vdim - 1]);
+          }
+        }
+#pragma unroll
+        for (int b = 0; b < kAhead; ++b) {
+          const int key = j0 + b * KPI + vgroup;
+          const float p = key < kWave ? m_s[wave][key] : 0.f;
+#pragma unroll
+          for (int i = 0; i < VPL; ++i) acc[s][i] = fmaf(p, vv[b][i], acc[s][i]);
+        }
+      }
+      wave_sync();
+    }
+    __syncthreads();                                        // before the next tile's weights take their place
+  }
+  const bool writer = !LPK || lane < LPK;                   // (the other lanes hold copies)
+#pragma unroll
+  for (int s = 0; s < SL; ++s) {
+    const int h = wave + s * n_waves;
+    if (h >= n_heads) break;
+    float g = 1.0f;
+    if (gate) {
+      const long at = row * gate_row + h;
+      const float z = gate_dtype == kF32 ? static_cast<const float*>(gate)[at] : to_float(static_cast<const bf16_t*>(gate)[at]);
+      g = 1.0f / (1.0f + expf(-z));
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      float r = acc[s][i];
+      if (LPK && LPK < kWave) {                             // the groups of lanes that took different keys: their sums together
+        if (LPK <= 16) r += __shfl_xor(r, 16, kWave);
+        r += __shfl_xor(r, 32, kWave);
+      }
+      const int c = vcol[i];
+      if (c >= vdim || !writer) continue;
+      const long at = (static_cast<long>(row) * n_heads + h) * vdim + c;
+      if (out_dtype == kF32) static_cast<float*>(out)[at] = r * g;
+      else static_cast<bf16_t*>(out)[at] = from_float<bf16_t>(r * g);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace bc4g
+
+using namespace bc4g;
+
+extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
+                                   const int32_t* block_table, int table_stride, const int32_t* row_seq,
+                                   const int32_t* positions, const float* sink, const float* far1, const float* far2,
+                                   const float* talk, const void* gate, int gate_dtype, long gate_row, void* out,
+                                   int out_dtype, int n_rows, int n_heads, int n_kv_heads, int dim, int vdim,
+                                   int page_tokens, int window, float scale, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= kMaxHeads && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+               "attention_talk: bad sizes T=%d heads=%d/%d (at most %d heads)", n_rows, n_heads, n_kv_heads, kMaxHeads);
+  BC4G_REQUIRE(dim > 0 && dim <= kMaxDim && vdim > 0 && vdim <= kMaxVdim, "attention_talk: dim=%d (at most %d), vdim=%d (at most %d)",
+               dim, kMaxDim, vdim, kMaxVdim);
+  const int e4 = dim <= 64 ? 2 : 8;
+  BC4G_REQUIRE(n_heads * 32 * e4 <= kMaxQ, "attention_talk: %d heads of %d are more than the %d numbers a row's queries may take",
+               n_heads, dim, kMaxQ);
+  BC4G_REQUIRE(page_tokens > 0 && table_stride > 0 && window >= 0, "attention_talk: bad cache sizes page_tokens=%d table_stride=%d window=%d",
+               page_tokens, table_stride, window);
+  BC4G_REQUIRE(q && k_cache && v_cache && block_table && row_seq && positions && out && q_row >= static_cast<long>(n_heads) * dim &&
+               (!gate || gate_row >= n_heads) && (out_dtype == kF32 || out_dtype == kBF16) &&
+               (!gate || gate_dtype == kF32 || gate_dtype == kBF16) && (far1 == nullptr) == (far2 == nullptr),
+               "attention_talk: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int waves = n_heads < kMaxWaves ? n_heads : kMaxWaves;
+  const int slots = (n_heads + waves - 1) / waves;
+  const size_t lds = static_cast<size_t>(n_heads) * (32 * e4 + kWave) * sizeof(float);
+  const bool v_four = vdim % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+#define BC4G_TALK(T, SL, E, V)                                                                                              \
+  attention_talk_kernel<T, SL, E, V><<<n_rows, waves * kWave, lds, s>>>(                                                    \
+      q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table, table_stride, row_seq, positions, \
+      sink, far1, far2, talk, gate, gate_dtype, gate_row, out, out_dtype, n_heads, n_kv_heads, dim, vdim, page_tokens, window, \
+      scale)
+#define BC4G_TALK_V(T, SL, E)                                                                                               \
+  do { if (!v_four) BC4G_TALK(T, SL, E, 0); else if (vdim <= 64) BC4G_TALK(T, SL, E, 16); else if (vdim <= 128) BC4G_TALK(T, SL, E, 32); else BC4G_TALK(T, SL, E, 64); } while (0)
+#define BC4G_TALK_E(T, SL)                                                                                                  \
+  do { if (e4 == 2) BC4G_TALK_V(T, SL, 2); else BC4G_TALK_V(T, SL, 8); } while (0)
+#define BC4G_TALK_S(T)                                                                                                      \
+  do { if (slots <= 1) BC4G_TALK_E(T, 1); else if (slots <= 2) BC4G_TALK_E(T, 2); else if (slots <= 4) BC4G_TALK_E(T, 4); else BC4G_TALK_E(T, 8); } while (0)
+  if (cache_dtype == kF32) BC4G_TALK_S(float);
+  else if (cache_dtype == kBF16) BC4G_TALK_S(bf16_t);
+  else return fail("attention_talk: unknown dtype %d", cache_dtype);
+#undef BC4G_TALK
+#undef BC4G_TALK_V
+#undef BC4G_TALK_E
+#undef BC4G_TALK_S
+  return check_launch("attention_talk");
+}

@@ -6,8 +6,9 @@
 //   rotation  a table of cosines and sines of position * frequency for the rotate-half pairing (element i with element
 //             i + half), the frequencies given by the caller (so any scaling of them is the caller's), both multiplied
 //             by an amplitude; angles in double.
-//   prepare   per (row, head): + bias, RMS norm over the head with a weight, rotation, a factor -- each optional -- into
-//             a dense tensor or into the pages of a cache.
+//   prepare   per (row, head): + bias, RMS norm over the head with a weight, rotation (either pairing), division by the
+//             root mean square after the rotation, a factor -- each optional -- into a dense tensor or into the pages
+//             of a cache.
 //   finish    per (row, head): o / rms(o) (* weight) * factor * act(gate).
 //
 // The scan walks a request's rows in chunks of 32, each chunk by workgroups of its own (a thread keeps one column of
@@ -81,19 +82,35 @@ __global__ __launch_bounds__(kWave) void heads_prepare_kernel(const PrepareSecti
   } else {
     base = row * p.out_row + static_cast<long>(head) * dim;
   }
-  for (int c = lane; c < dim; c += kWave) {
-    float v;
-    if (c < 2 * half) {
-      const int i = c < half ? c : c - half;
-      float lo = vals[i] * scale, hi = vals[i + half] * scale;
-      if (norm_w) lo *= norm_w[i], hi *= norm_w[i + half];
-      const float cs = table[(static_cast<long>(row) * half + i) * 2], sn = table[(static_cast<long>(row) * half + i) * 2 + 1];
-      v = c < half ? lo * cs - hi * sn : hi * cs + lo * sn;
-    } else {
-      v = vals[c] * scale;
-      if (norm_w) v *= norm_w[c];
+  float turned[kMaxHead / kWave];      // this lane's elements after norm and rotation
+  float ss_after = 0.f;
+#pragma unroll
+  for (int n = 0; n < kMaxHead / kWave; ++n) {
+    const int c = lane + n * kWave;
+    float v = 0.f;
+    if (c < dim) {
+      if (c < 2 * half) {
+        // the pair's two members: element i with element i + half, or (neighbours) element 2i with element 2i + 1
+        const int i = p.pairing ? c / 2 : (c < half ? c : c - half);
+        const int at_lo = p.pairing ? 2 * i : i, at_hi = p.pairing ? 2 * i + 1 : i + half;
+        float lo = vals[at_lo] * scale, hi = vals[at_hi] * scale;
+        if (norm_w) lo *= norm_w[at_lo], hi *= norm_w[at_hi];
+        const float cs = table[(static_cast<long>(row) * half + i) * 2], sn = table[(static_cast<long>(row) * half + i) * 2 + 1];
+        v = c == at_lo ? lo * cs - hi * sn : hi * cs + lo * sn;
+      } else {
+        v = vals[c] * scale;
+        if (norm_w) v *= norm_w[c];
+      }
     }
-    store_any(p.out, p.out_dtype, base + c, v * p.factor);
+    turned[n] = v;
+    ss_after = fmaf(v, v, ss_after);
+  }
+  // (unit_after: the head divided by its root mean square as it stands after the rotation, no weight)
+  const float last = p.unit_after ? p.factor / sqrtf(wave_sum(ss_after) / static_cast<float>(dim) + p.eps) : p.factor;
+#pragma unroll
+  for (int n = 0; n < kMaxHead / kWave; ++n) {
+    const int c = lane + n * kWave;
+    if (c < dim) store_any(p.out, p.out_dtype, base + c, turned[n] * last);
   }
 }
 

@@ -17,11 +17,15 @@ constexpr int kBlock = 256;
 // ---- embedding -------------------------------------------------------------
 template <typename TT>
 __global__ void embed_gather_kernel(const TT* __restrict__ table, const int32_t* __restrict__ ids,
-                                    float* __restrict__ out, int hidden) {
+                                    float* __restrict__ out, int hidden, int add) {
   const size_t row = blockIdx.x;
   const TT* src = table + static_cast<size_t>(ids[row]) * hidden;
   float* dst = out + row * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+  if (add) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(src[i]);
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+  }
 }
 
 // ---- RMSNorm ---------------------------------------------------------------
@@ -613,20 +617,30 @@ int grid_for(long total) {
 
 using namespace bc4g;
 
-extern "C" int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
-                                 int n_tokens, int hidden, int vocab, void* stream) {
-  BC4G_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d",
+static int embed_rows(const char* what, const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens,
+                      int hidden, int vocab, int add, void* stream) {
+  BC4G_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0 && table && ids && out, "%s: bad arguments T=%d H=%d V=%d", what,
                n_tokens, hidden, vocab);
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (table_dtype == kF32) {
-    embed_gather_kernel<float><<<n_tokens, kBlock, 0, s>>>(static_cast<const float*>(table), ids, out, hidden);
+    embed_gather_kernel<float><<<n_tokens, kBlock, 0, s>>>(static_cast<const float*>(table), ids, out, hidden, add);
   } else if (table_dtype == kBF16) {
-    embed_gather_kernel<bf16_t><<<n_tokens, kBlock, 0, s>>>(static_cast<const bf16_t*>(table), ids, out, hidden);
+    embed_gather_kernel<bf16_t><<<n_tokens, kBlock, 0, s>>>(static_cast<const bf16_t*>(table), ids, out, hidden, add);
   } else {
-    return fail("embed_gather: unknown table dtype %d", table_dtype);
+    return fail("%s: unknown table dtype %d", what, table_dtype);
   }
-  return check_launch("embed_gather");
+  return check_launch(what);
+}
+
+extern "C" int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
+                                 int n_tokens, int hidden, int vocab, void* stream) {
+  return embed_rows("embed_gather", table, table_dtype, ids, out, n_tokens, hidden, vocab, 0, stream);
+}
+
+extern "C" int bc4g_embed_add(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
+                              int vocab, void* stream) {
+  return embed_rows("embed_add", table, table_dtype, ids, out, n_tokens, hidden, vocab, 1, stream);
 }
 
 extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,

@@ -99,6 +99,16 @@ __global__ void clamped_glu_pieces_kernel(const bf16_t* __restrict__ gu, bf16_t*
   }
 }
 
+// z Phi(z), the exact gelu: 0.5 z (1 + erf(z / sqrt 2)).
+template <typename T>
+__global__ void gelu_kernel(const T* __restrict__ in, T* __restrict__ out, long total) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total; i += stride) {
+    const float z = to_float(in[i]);
+    out[i] = from_float<T>(0.5f * z * (1.0f + erff(z * 0.70710678118654752440f)));
+  }
+}
+
 int grid_for(long total) {
   const long g = (total + kBlock - 1) / kBlock;
   return static_cast<int>(g < 1 ? 1 : (g > 65535 ? 65535 : g));
@@ -143,4 +153,14 @@ extern "C" int bc4g_clamped_glu(const void* gu, void* out, int dtype, float limi
   else if (dtype == kBF16) clamped_glu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), limit, slope, total, inter);
   else return fail("clamped_glu: unknown dtype %d", dtype);
   return check_launch("clamped_glu");
+}
+
+extern "C" int bc4g_gelu(const void* in, void* out, int dtype, long total, void* stream) {
+  BC4G_REQUIRE(total >= 0 && in && out, "gelu: bad arguments total=%ld", total);
+  if (total == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32) gelu_kernel<float><<<grid_for(total), kBlock, 0, s>>>(static_cast<const float*>(in), static_cast<float*>(out), total);
+  else if (dtype == kBF16) gelu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), total);
+  else return fail("gelu: unknown dtype %d", dtype);
+  return check_launch("gelu");
 }

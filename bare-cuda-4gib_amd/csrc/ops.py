@@ -99,6 +99,19 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Ten
     return out
 
 
+def embed_add(table: torch.Tensor, ids: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """x[t, :] += float(table[ids[t], :]) in place on the float32 stream x [T, H]."""
+    _dev("embed_add", table, ids, x)
+    vocab, hidden = table.shape
+    n = ids.numel()
+    _i32("embed_add", "ids", ids, n)
+    if x.dtype != torch.float32 or tuple(x.shape) != (n, hidden) or not x.is_contiguous():
+        raise KernelError(f"embed_add: x must be float32 [{n}, {hidden}], got {x.dtype} {tuple(x.shape)}")
+    library.call("bc4g_embed_add", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, _stream(),
+                 cost=lambda: (1.0 * n * hidden, n * hidden * (table.element_size() + 8)))
+    return x
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
     """RMSNorm of rows of the float residual stream x [T, H]; with ``rows`` (int32
@@ -1516,15 +1529,18 @@ class _PrepareSection(ctypes.Structure):
                 ("out", ctypes.c_void_p), ("slot_map", ctypes.c_void_p), ("in_row", ctypes.c_long), ("out_row", ctypes.c_long),
                 ("page_stride", ctypes.c_long), ("head_stride", ctypes.c_long), ("token_stride", ctypes.c_long),
                 ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int), ("half", ctypes.c_int), ("page_tokens", ctypes.c_int),
-                ("heads", ctypes.c_int), ("dim", ctypes.c_int), ("eps", ctypes.c_float), ("factor", ctypes.c_float)]
+                ("heads", ctypes.c_int), ("dim", ctypes.c_int), ("eps", ctypes.c_float), ("factor", ctypes.c_float),
+                ("pairing", ctypes.c_int), ("unit_after", ctypes.c_int)]
 
 
 def heads_section(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                   norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, table: Optional[torch.Tensor] = None,
-                  factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0):
+                  factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0,
+                  neighbours: bool = False, unit_after: bool = False):
     """One section for heads_prepare_many: every head of x [T, heads * dim] (may be a part of wider rows): + bias, RMS norm
-    over the head with ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half), times
-    ``factor``.  ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache
+    over the head with ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half, or with
+    ``neighbours`` element 2i with element 2i + 1), with ``unit_after`` division by sqrt(mean(head^2) + eps) of the head as
+    it stands then, times ``factor``.  ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache
     [pages, heads, page_tokens, dim] whose slot page * page_tokens + offset receives the row.  Checked here; the tensors
     must live until the launch."""
     _dev("heads_prepare", bias, norm_weight, table, out, slot_map)
@@ -1550,7 +1566,7 @@ def heads_section(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, b
         out_row = heads * dim
     section = _PrepareSection(_ptr(x), _ptr(bias), _ptr(norm_weight), _ptr(table), _ptr(out), _ptr(slot_map), in_row, out_row,
                               page_stride, head_stride, token_stride, _code(x, "heads_prepare"), _code(out, "heads_prepare"), half,
-                              page_tokens, heads, dim, float(eps), float(factor))
+                              page_tokens, heads, dim, float(eps), float(factor), 1 if neighbours else 0, 1 if unit_after else 0)
     return section, t, t * heads * dim, x.element_size() + out.element_size()
 
 
@@ -1651,14 +1667,19 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.T
 def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
                    n_heads: int, n_kv_heads: int, maps: int, dim: int, vdim: int, window: int, keep_first: int, scale: float, *,
                    lam: float = 0.0, normalize: bool = False, eps: float = 0.0, factor: float = 1.0,
-                   gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID, waves: int = 0) -> torch.Tensor:
+                   gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID, waves: int = 0,
+                   sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
     """Softmax attention with ``maps`` (1 or 2) score maps per query head over the same values: q float32
     [T, n_heads, maps, dim]; keys [pages, n_kv_heads * maps, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].
     A row at position p sees key j <= p if p - j < window or j < keep_first (window 0: every key).  o = a1 - lam a2,
     with ``normalize`` divided by sqrt(mean(o^2) + eps) over the head, times ``factor`` and act(gate); [T, n_heads * vdim].
     ``waves``: how many waves cut one row's keys among them (0: chosen here -- one where the rows fill the GPU, up to
-    eight where few rows walk long contexts)."""
-    _dev("attention_maps", q, k_cache, v_cache, block_table)
+    eight where few rows walk long contexts).  ``sink`` (float32 [n_heads]): exp(sink) joins every map's denominator, with
+    no key and no value.  ``far`` = (r1, r2), float32 [n_heads] each: r1 ln(1 + r2 (p - j)) is taken off the scaled score."""
+    _dev("attention_maps", q, k_cache, v_cache, block_table, sink, *(far or ()))
+    _f32("attention_maps", "sink", sink, (n_heads,))
+    for v in far or ():
+        _f32("attention_maps", "far", v, (n_heads,))
     t = q.shape[0]
     if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, maps, dim):
         raise KernelError(f"attention_maps: q must be float32 [T, {n_heads}, {maps}, {dim}], got {q.dtype} {tuple(q.shape)}")
@@ -1695,5 +1716,134 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                  _ptr(block_table), block_table.stride(0), _ptr(ctx.row_seq), _ptr(ctx.positions), float(lam), 1 if normalize else 0,
                  float(eps), float(factor), _ptr(gate), _code(gate, "attention_maps") if gate is not None else F32, gate_row, int(act),
                  _ptr(out), _code(out, "attention_maps"), t, n_heads, n_kv_heads, maps, dim, vdim, page_tokens, int(window),
-                 int(keep_first), float(scale), int(waves), _stream(), cost=cost)
+                 int(keep_first), float(scale), int(waves), _ptr(sink), _ptr(far[0]) if far else None,
+                 _ptr(far[1]) if far else None, _stream(), cost=cost)
+    return out
+
+
+TALK_MAX_HEADS = 64          # query heads whose weights attention_talk mixes
+TALK_MAX_QUERIES = 8192      # heads * (dim rounded up: 64 up to 64, else 256) that a row's queries may take in its LDS
+
+
+def attention_talk_takes(n_heads: int, dim: int, vdim: int) -> bool:
+    return (0 < n_heads <= TALK_MAX_HEADS and 0 < dim <= HEADS_MAX_DIM and 0 < vdim <= HEADS_MAX_DIM
+            and n_heads * (64 if dim <= 64 else 256) <= TALK_MAX_QUERIES)
+
+
+def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
+                   n_heads: int, n_kv_heads: int, dim: int, vdim: int, window: int, scale: float, *,
+                   sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                   talk: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Windowed softmax attention whose heads' weights are mixed before they meet the values: q float32 [T, n_heads, dim];
+    keys [pages, n_kv_heads, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].  A row at position p sees key
+    j <= p with p - j < window (0: every key).  score = q . k * scale - r1 ln(1 + r2 (p - j)) (``far`` = (r1, r2));
+    w_g = exp(score_g) / (sum_j exp(score_g) + exp(sink_g)); head h weighs the values of its own key/value head by
+    sum_g talk[h, g] w_g (``talk`` float32 [n_heads, n_heads]; none: its own weights) and is multiplied by
+    sigmoid(gate[t, h]) (``gate`` [T, n_heads], may be a part of wider rows).  Returns [T, n_heads * vdim]."""
+    _dev("attention_talk", q, k_cache, v_cache, block_table, sink, talk, *(far or ()))
+    t = q.shape[0]
+    if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, dim) or not q.is_contiguous():
+        raise KernelError(f"attention_talk: q must be float32 [T, {n_heads}, {dim}], got {q.dtype} {tuple(q.shape)}")
+    if not attention_talk_takes(n_heads, dim, vdim):
+        raise KernelError(f"attention_talk: {n_heads} heads of {dim} with values of {vdim} are beyond the kernel")
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.dtype != v_cache.dtype:
+        raise KernelError("attention_talk: caches must be [pages, heads, page_tokens, size] of one dtype")
+    pages, _, page_tokens, _ = k_cache.shape
+    if tuple(k_cache.shape[1:]) != (n_kv_heads, page_tokens, dim) or tuple(v_cache.shape) != (pages, n_kv_heads, page_tokens, vdim):
+        raise KernelError(f"attention_talk: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit {n_kv_heads} key/value "
+                          f"heads, keys of {dim}, values of {vdim}")
+    if ctx.n_tokens != t or block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.shape[0] < ctx.n_seqs:
+        raise KernelError("attention_talk: the block table does not fit the step")
+    _i32("attention_talk", "row_seq", ctx.row_seq, t)
+    _i32("attention_talk", "positions", ctx.positions, t)
+    _f32("attention_talk", "sink", sink, (n_heads,))
+    _f32("attention_talk", "talk", talk, (n_heads, n_heads))
+    for v in far or ():
+        _f32("attention_talk", "far", v, (n_heads,))
+    gate_row = _part_of_rows("attention_talk", "gate", gate, n_heads) if gate is not None else 0
+    if gate is not None and gate.shape[0] != t:
+        raise KernelError(f"attention_talk: gate has {gate.shape[0]} rows, q {t}")
+    out = torch.empty((t, n_heads * vdim), dtype=out_dtype, device=q.device)
+
+    def cost():
+        keys = pairs = 0
+        for s in range(ctx.n_seqs):
+            cached, new = int(ctx.seq_ctx[s]), int(ctx.seq_start[s + 1] - ctx.seq_start[s])
+            if window > 0:
+                pairs += sum(min(window, cached + i + 1) for i in range(new))
+                keys += min(cached + new, window + new - 1)
+            else:
+                pairs += new * cached + new * (new + 1) // 2
+                keys += cached + new
+        mixing = n_heads if talk is not None else 0
+        return (2.0 * pairs * n_heads * (dim + vdim + mixing),
+                keys * n_kv_heads * (dim + vdim) * k_cache.element_size() + t * n_heads * (4 * dim + vdim * out.element_size()))
+    library.call("bc4g_attention_talk", _ptr(q), n_heads * dim, _ptr(k_cache), _ptr(v_cache), _code(k_cache, "attention_talk"),
+                 _ptr(block_table), block_table.stride(0), _ptr(ctx.row_seq), _ptr(ctx.positions), _ptr(sink),
+                 _ptr(far[0]) if far else None, _ptr(far[1]) if far else None, _ptr(talk), _ptr(gate),
+                 _code(gate, "attention_talk") if gate is not None else F32, gate_row, _ptr(out), _code(out, "attention_talk"),
+                 t, n_heads, n_kv_heads, dim, vdim, page_tokens, int(window), float(scale), _stream(), cost=cost)
+    return out
+
+
+# ---- activations and routing of a mixture of experts ------------------------------------------------------------------------
+
+def gelu(z: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """z Phi(z), the exact gelu, element by element; ``out`` may be z itself."""
+    _dev("gelu", z, out)
+    if not z.is_contiguous():
+        raise KernelError("gelu: the input's elements must lie side by side")
+    if out is None:
+        out = torch.empty_like(z)
+    elif out.dtype != z.dtype or out.shape != z.shape or not out.is_contiguous():
+        raise KernelError("gelu: out must have the input's dtype and shape")
+    total = z.numel()
+    library.call("bc4g_gelu", _ptr(z), _ptr(out), _code(z, "gelu"), total, _stream(),
+                 cost=lambda: (10.0 * total, 2 * total * z.element_size()))
+    return out
+
+
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(logits: torch.Tensor, experts: int, top: int, groups: int = 1, keep: int = 1,
+              correction: Optional[torch.Tensor] = None, want_chosen: bool = False):
+    """The choice of experts for every row: logits float32 [T, >= experts] (the first ``experts`` columns count; rows may
+    be parts of wider rows).  s = softmax(logits); the choice goes by s + correction; only experts of the ``keep`` best of
+    ``groups`` equal groups of neighbours (a group counts by its largest choice) can be chosen; the ``top`` largest win.
+    Returns weights float32 [T, experts] -- s of the chosen, zero elsewhere -- and, if asked, the chosen int32 [T, top]."""
+    _dev("moe_route", correction)
+    row = _part_of_rows("moe_route", "logits", logits, experts)
+    if logits.dtype != torch.float32:
+        raise KernelError(f"moe_route: logits must be float32, got {logits.dtype}")
+    _f32("moe_route", "correction", correction, (experts,))
+    t = logits.shape[0]
+    weights = torch.empty((t, experts), dtype=torch.float32, device=logits.device)
+    chosen = torch.empty((t, top), dtype=torch.int32, device=logits.device) if want_chosen else None
+    library.call("bc4g_moe_route", _ptr(logits), row, _ptr(correction), _ptr(weights), _ptr(chosen), t, experts, groups, keep, top,
+                 _stream(), cost=lambda: (8.0 * t * experts * (1 + top), 8.0 * t * experts))
+    return (weights, chosen) if want_chosen else weights
+
+
+def routed_glu(gu: torch.Tensor, weights: Optional[torch.Tensor], experts: int, ff: int, limit: float, *, shared_ff: int = 0,
+               shared_limit: float = 0.0, shared_logit: Optional[torch.Tensor] = None, slope: float = 1.702) -> torch.Tensor:
+    """gu [T, experts * 2 ff + 2 shared_ff]: per expert its ff gates, then its ff ups, and last the shared unit's.  Returns
+    [T, experts * ff + shared_ff]: weights[t, e] * g sigmoid(slope g) (u + 1) with g = min(gate, limit),
+    u = clamp(up, -limit, limit); the shared unit (its own limit) times sigmoid(shared_logit[t]) (float32 [T, 1], may be a
+    part of wider rows)."""
+    _dev("routed_glu", gu, weights)
+    t = gu.shape[0]
+    if gu.dim() != 2 or gu.shape[1] != 2 * (experts * ff + shared_ff) or not gu.is_contiguous():
+        raise KernelError(f"routed_glu: input must be [T, {2 * (experts * ff + shared_ff)}], got {tuple(gu.shape)}")
+    if experts:
+        _f32("routed_glu", "weights", weights, (t, experts))
+    shared_row = 0
+    if shared_ff:
+        if shared_logit is None or shared_logit.dtype != torch.float32 or shared_logit.shape[0] != t:
+            raise KernelError("routed_glu: the shared unit needs a float32 gate logit for every row")
+        shared_row = _part_of_rows("routed_glu", "shared_logit", shared_logit, 1)
+    out = torch.empty((t, experts * ff + shared_ff), dtype=gu.dtype, device=gu.device)
+    library.call("bc4g_routed_glu", _ptr(gu), _ptr(out), _code(gu, "routed_glu"), _ptr(weights), _ptr(shared_logit), shared_row,
+                 float(limit), float(shared_limit), float(slope), t, experts, ff, shared_ff, _stream(),
+                 cost=lambda: (8.0 * out.numel(), 3 * out.numel() * gu.element_size()))
     return out

@@ -55,6 +55,10 @@ class Model:
         for e in self.schedule:
             if not (0 <= e.layer < len(self.layers)):
                 raise ConfigError(f"schedule names layer {e.layer}, the model has {len(self.layers)}")
+            if getattr(e, "add_embedding", False) and (int(getattr(spec, "streams", 1)) != 1
+                                                       or not hasattr(self.embedding.part, "add_to")):
+                raise ConfigError("a schedule entry adds the embedding to the stream: that takes one copy of the stream and "
+                                  "an embedding part that can add")
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
         self.max_seq_len = spec.max_seq_len
@@ -157,6 +161,9 @@ class Model:
         the live requests, as the parts state them; a layer that the schedule names twice counts twice."""
         flops, nbytes = self.embedding.part.step_work(batch, batch.n_tokens, elem)
         for e in self.schedule:
+            if e.add_embedding:
+                f, b = self.embedding.part.step_work(batch, batch.n_tokens, elem)
+                flops, nbytes = flops + f, nbytes + b
             f, b = self.layers[e.layer].step_work(batch, batch.n_tokens, elem)
             flops, nbytes = flops + f, nbytes + b
         for part in (self.final_norm.part, self.head.part):
@@ -184,8 +191,12 @@ class Model:
         ctx.handoff.end_step()
         for i, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
-            following = self.layers[self.schedule[i + 1].layer] if i + 1 < len(self.schedule) else None
+            # (nobody prepares the first norm of an entry before which the stream changes once more)
+            following = (self.layers[self.schedule[i + 1].layer]
+                         if i + 1 < len(self.schedule) and not self.schedule[i + 1].add_embedding else None)
             ctx.handoff.begin_entry(layer, following, ctx.n_tokens)
+            if e.add_embedding:
+                self.embedding.part.add_to(x, ctx)
             layer.forward(x, ctx, ctx.cache(e.cache), e.writes)
         ctx.handoff.end_step()
         if ctx.n_logits == 0:

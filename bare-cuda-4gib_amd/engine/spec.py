@@ -40,10 +40,13 @@ class ScheduleEntry:
     """One execution of a layer.  ``cache`` names the cache stream its mixer
     uses (any hashable id; entries that share an id share the cache), and
     ``writes`` says whether this execution appends to that stream or only
-    reads what another entry wrote."""
+    reads what another entry wrote.  ``add_embedding``: the embedding's output is added to the
+    residual stream right before this execution (a stack that runs some of its layers several times
+    feeds its input in again at the start of every further pass)."""
     layer: int
     cache: Optional[Any] = None
     writes: bool = True
+    add_embedding: bool = False
 
 
 @dataclasses.dataclass

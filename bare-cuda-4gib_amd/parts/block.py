@@ -12,22 +12,38 @@ from .streams import StreamReader
 
 class PreNormBlock(Part):
     """x += mixer(norm(x)); x += ffn(norm(x))  (reference: engine/src/model.cpp:526-604).
-    The residual stream x is float32 and is updated in place."""
+    The residual stream x is float32 and is updated in place.  A layer may have no feed-forward, and the mixer may read
+    its input through a part that mixes every row with the row before it (``mixer_shift``, a conv part with a state of
+    its own: the layer then keeps that state beside its mixer's cache)."""
     category = "block"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
-    def __init__(self, mixer, ffn, mixer_norm, ffn_norm):
-        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm = mixer, ffn, mixer_norm, ffn_norm
+    def __init__(self, mixer, ffn, mixer_norm, ffn_norm, mixer_shift=None):
+        self.mixer, self.ffn, self.mixer_norm, self.ffn_norm, self.mixer_shift = mixer, ffn, mixer_norm, ffn_norm, mixer_shift
 
     def children(self):
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+        return [p for p in (self.mixer_norm, self.mixer_shift, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+
+    def cache_spec(self):
+        """The mixer's cache, and beside it the state of the shift in front of the mixer."""
+        if self.mixer_shift is None:
+            return self.mixer.cache_spec()
+        return Bundle((("mixer", self.mixer.cache_spec()), ("shift", self.mixer_shift.cache_spec())))
 
     def forward(self, x, ctx, cache, writes: bool = True) -> None:
         # Each part is told which norm reads the stream after it, so that its last product can prepare that
         # norm: the feed-forward's after the mixer, the next entry's first after the feed-forward.
         handoff, n = ctx.handoff, x.shape[0]
-        with handoff.reader(self.ffn_norm, self._wants_prepared(self.ffn, n)):
-            self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+        after_mixer = (self.ffn_norm, self._wants_prepared(self.ffn, n)) if self.ffn is not None else (handoff.next_entry or (None, False))
+        with handoff.reader(*after_mixer):
+            if self.mixer_shift is not None:
+                pre = handoff.take(self.mixer_norm)
+                h = pre.tensor if isinstance(pre, ops.Finished) else self.mixer_norm.forward(x, ctx)
+                self.mixer.forward(self.mixer_shift.forward(h, ctx, cache.shift), ctx, cache.mixer, x, writes)
+            else:
+                self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+        if self.ffn is None:
+            return
         with handoff.reader(*(handoff.next_entry or (None, False))):
             self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
 

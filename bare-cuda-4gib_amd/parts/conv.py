@@ -44,4 +44,32 @@ class CausalConv(Part):
                                add_input=add_input)
 
 
+class TokenShift(Part):
+    """out[t] = h[t] + (h[t - 1] - h[t]) * m, element by element, along a request's rows; h[-1] = 0.  The h on the right
+    are the rows as they came in.  A request's last row is its state (``tail``, in the activations' dtype), so a prompt
+    may be cut anywhere.  It is the causal convolution with the taps (m, -m) plus its input."""
+    category = "conv"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+
+    def __init__(self, channels: int):
+        if channels <= 0:
+            raise ConfigError(f"token shift: {channels} channels")
+        self.channels = int(channels)
+        self.w = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {"weight": WeightSpec((self.channels,), kind="vector")}
+
+    def bind(self, tensors, rt) -> None:
+        m = tensors["weight"].to(torch.float32)
+        self.w = torch.stack([m, -m], dim=0).contiguous()      # by taps: the row before, the row itself
+
+    def cache_spec(self):
+        return States((("tail", (1, self.channels), None),))
+
+    def forward(self, h: torch.Tensor, ctx, view) -> torch.Tensor:
+        return ops.causal_conv(h, self.w, view.tail, ctx, add_input=True)
+
+
 register_part("conv", "causal", CausalConv)
+register_part("conv", "token_shift", TokenShift)

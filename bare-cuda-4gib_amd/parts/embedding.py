@@ -30,6 +30,10 @@ class Embedding(Part):
     def forward(self, ctx) -> torch.Tensor:
         return ops.embed_gather(self.table, ctx.token_ids)
 
+    def add_to(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        """x += the embedding of the step's tokens, in place on the float32 stream."""
+        return ops.embed_add(self.table, ctx.token_ids, x)
+
 
 class LMHead(Part):
     """logits = h W^T in float32 (reference: engine/src/model.cpp:612-615).  If

@@ -6,6 +6,7 @@ from typing import Dict
 import torch
 
 from ..csrc import ops
+from ..errors import ConfigError
 from ..weights.loader import WeightSpec
 from .base import Part, register_part
 from .linear import linear, linear_swiglu
@@ -111,6 +112,115 @@ class ClampedGLU(Part):
         linear(ops.clamped_glu(gu, self.limit, self.slope), self.w_down, accumulate_into=residual, ctx=ctx)
 
 
+class DenseGELU(Part):
+    """x += Wd gelu(Wu h), no biases, with the exact gelu z Phi(z)."""
+    category = "feedforward"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+    accepts_lazy_norm = True
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.w_up = self.w_down = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {"up": WeightSpec((i, h)), "down": WeightSpec((h, i))}
+
+    def bind(self, tensors, rt) -> None:
+        self.w_up = ops.StreamedWeight(tensors["up"])
+        self.w_down = ops.StreamedWeight(tensors["down"])
+        self.act_dtype = rt.act_dtype
+
+    def step_work(self, batch, rows: int, elem: int):
+        flops, nbytes = super().step_work(batch, rows, elem)
+        return flops + 10.0 * rows * self.intermediate_size, nbytes
+
+    def forward(self, h, ctx, residual) -> None:
+        z = linear(h, self.w_up, out_dtype=self.act_dtype)
+        linear(ops.gelu(z, out=z), self.w_down, accumulate_into=residual, ctx=ctx)
+
+
+class RoutedExperts(Part):
+    """A mixture of clamped gated units: x += sum over the chosen experts e of s_e * expert_e(h), plus, if there is one, a
+    shared expert for every row times sigmoid(Wsg h).
+
+    The router: z = Wr h in float32, s = softmax(z) over all experts; the choice goes by s + ``correction``; the experts
+    lie in ``groups`` equal groups of neighbours, a group counts by its largest choice, and only experts of the ``keep``
+    best groups can be chosen; the ``top`` largest choices win.  The weights are the chosen experts' s, as they are.
+    An expert: Wd (g sigmoid(slope g) (u + 1)) with g = min(Wg h, limit), u = clamp(Wu h, -limit, limit), no biases.
+
+    All experts' gate and up matrices are one product and all their down matrices another: between the two, a row's
+    units of the experts it did not choose are multiplied by zero and those of the chosen by their weights, so that the
+    second product adds up the weighted sum (the router's and the shared gate's logits are one small float32 product).
+    Tensors: ``router`` [experts, hidden], ``correction`` [experts], ``e<i>.{gate,up,down}``, ``shared.{gate,up,down}``,
+    ``shared.sg`` [1, hidden]."""
+    category = "feedforward"
+    graph_safe = True     # launches kernels only: may run inside a captured graph
+    accepts_lazy_norm = True
+    adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
+
+    def __init__(self, hidden_size: int, experts: int, top: int, intermediate_size: int, limit: float, groups: int = 1,
+                 keep: int = 1, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0, slope: float = 1.702):
+        self.hidden_size, self.experts, self.top, self.ff = int(hidden_size), int(experts), int(top), int(intermediate_size)
+        self.limit, self.groups, self.keep, self.correction = float(limit), int(groups), int(keep), bool(correction)
+        self.shared_ff, self.shared_limit, self.slope = int(shared_size), float(shared_limit), float(slope)
+        if not (0 < self.experts <= ops.MOE_MAX_EXPERTS) or not (0 < self.top <= self.experts) or self.ff <= 0:
+            raise ConfigError(f"routed experts: {self.top} of {self.experts} experts (at most {ops.MOE_MAX_EXPERTS}) of size {self.ff}")
+        if self.groups <= 0 or self.experts % self.groups or not (0 < self.keep <= self.groups):
+            raise ConfigError(f"routed experts: {self.experts} experts in {self.groups} groups of which {self.keep} are kept")
+        if self.top > self.keep * (self.experts // self.groups):
+            raise ConfigError(f"routed experts: {self.top} experts cannot be chosen from {self.keep} groups of "
+                              f"{self.experts // self.groups}")
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, f = self.hidden_size, self.ff
+        out = {"router": WeightSpec((self.experts, h))}
+        if self.correction:
+            out["correction"] = WeightSpec((self.experts,), kind="vector")
+        for e in range(self.experts):
+            out.update({f"e{e}.gate": WeightSpec((f, h)), f"e{e}.up": WeightSpec((f, h)), f"e{e}.down": WeightSpec((h, f))})
+        if self.shared_ff:
+            g = self.shared_ff
+            out.update({"shared.gate": WeightSpec((g, h)), "shared.up": WeightSpec((g, h)), "shared.down": WeightSpec((h, g)),
+                        "shared.sg": WeightSpec((1, h))})
+        return out
+
+    def bind(self, tensors, rt) -> None:
+        names = [f"e{e}" for e in range(self.experts)] + (["shared"] if self.shared_ff else [])
+        # per expert its gates' rows, then its ups'; the down matrices side by side along their inputs
+        self.w_gu = ops.StreamedWeight(torch.cat([tensors[f"{n}.{part}"] for n in names for part in ("gate", "up")], dim=0).contiguous())
+        self.w_down = ops.StreamedWeight(torch.cat([tensors[f"{n}.down"] for n in names], dim=1).contiguous())
+        self.w_route = ops.StreamedWeight(torch.cat([tensors["router"]] + ([tensors["shared.sg"]] if self.shared_ff else []),
+                                                    dim=0).contiguous())
+        self.correction_w = tensors["correction"].to(torch.float32).contiguous() if self.correction else None
+        self.act_dtype = rt.act_dtype
+
+    def step_work(self, batch, rows: int, elem: int):
+        """What the design asks for: the router, ``top`` experts a row and the shared one; every weight read once."""
+        h = self.hidden_size
+        units = self.top * self.ff + self.shared_ff
+        flops = 2.0 * rows * h * (self.experts + (1 if self.shared_ff else 0)) + rows * units * (6.0 * h + 8.0)
+        nbytes = (self.experts * (3 * self.ff * h + h) + (3 * self.shared_ff * h + h if self.shared_ff else 0)) * elem
+        return flops, float(nbytes)
+
+    def working_bytes_per_row(self, elem: int) -> float:
+        return 3.0 * (self.experts * self.ff + self.shared_ff) * elem + 8.0 * (self.experts + 1)
+
+    def forward(self, h, ctx, residual) -> None:
+        if hasattr(h, "tensor") and callable(h.tensor):      # (three products read the norm: it is computed once)
+            h = h.tensor()
+        E = self.experts
+        z = linear(h, self.w_route, out_dtype=torch.float32)
+        weights = ops.moe_route(z, E, self.top, self.groups, self.keep, self.correction_w)
+        gu = linear(h, self.w_gu, out_dtype=self.act_dtype)
+        y = ops.routed_glu(gu, weights, E, self.ff, self.limit, shared_ff=self.shared_ff, shared_limit=self.shared_limit,
+                           shared_logit=z[:, E:E + 1] if self.shared_ff else None, slope=self.slope)
+        linear(y, self.w_down, accumulate_into=residual, ctx=ctx)
+
+
 register_part("feedforward", "swiglu", SwiGLU)
+register_part("feedforward", "dense_gelu", DenseGELU)
+register_part("feedforward", "routed_experts", RoutedExperts)
 register_part("feedforward", "clamped_glu", ClampedGLU)
 register_part("feedforward", "dense_xielu", DenseXIELU)

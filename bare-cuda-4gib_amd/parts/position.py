@@ -18,11 +18,17 @@ class Rotary(Part):
     e(t) = dim ln(L / (2 pi t)) / (2 ln theta), lo = max(floor(e(fast)), 0), hi = min(ceil(e(slow)), dim - 1) and
     r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns with inv_freq_i / F * r_i + inv_freq_i (1 - r_i), and
     cosines and sines are multiplied by 0.1 ln F + 1.  The kernels that rotate inside a product take no scaling
-    (``fused()`` is None then); ``table(ctx)`` gives every row's cosines and sines to whoever rotates by a table."""
+    (``fused()`` is None then); ``table(ctx)`` gives every row's cosines and sines to whoever rotates by a table.
+
+    ``pairing`` "neighbours" turns element 2i with element 2i + 1 instead (the same angles, the same table); only
+    kernels that rotate by a table know that pairing."""
     category = "position"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
-    def __init__(self, theta: float, dim: int, scaling=None):
+    def __init__(self, theta: float, dim: int, scaling=None, pairing: str = "half"):
+        if pairing not in ("half", "neighbours"):
+            raise ConfigError(f"rotary: pairing must be 'half' or 'neighbours', got {pairing!r}")
+        self.pairing = pairing
         if dim <= 0 or dim % 2:
             raise ConfigError(f"rotary: dim must be positive and even, got {dim}")
         if theta <= 0:
@@ -39,10 +45,15 @@ class Rotary(Part):
         self._freqs = None
 
     def fused(self):
-        return (self.dim, self.theta) if self.scaling is None else None
+        return (self.dim, self.theta) if self.scaling is None and self.pairing == "half" else None
+
+    @property
+    def neighbours(self) -> bool:
+        return self.pairing == "neighbours"
 
     def apply(self, qkv, ctx, n_heads, n_kv_heads, head_dim):
-        raise ConfigError("rotary: scaled frequencies are applied by a table (table(ctx)); this mixer rotates inside its product")
+        raise ConfigError("rotary: scaled frequencies and neighbouring pairs are applied by a table (table(ctx)); this mixer "
+                          "rotates inside its product")
 
     def frequencies(self):
         """(what pair i turns by per position, for i < dim / 2, as Python floats; the factor on cosines and sines)."""
