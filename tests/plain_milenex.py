@@ -121,6 +121,25 @@ def route(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep
     return chosen, torch.gather(s, 1, chosen)
 
 
+def route_margin(z: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int) -> torch.Tensor:
+    """[T]: how far every row's choice is from another one -- the smaller of the gap between the last kept group's score
+    and the best group's left out, and the gap between the last chosen expert's choice score and the best one's left out
+    among the kept groups (infinite where nothing is left out).  A test in reduced precision knows by it which rows'
+    choice a rounding could turn."""
+    T, E = z.shape
+    choice = torch.softmax(z, dim=-1) + correction
+    per = E // groups
+    best = choice.view(T, groups, per).max(dim=-1).values.sort(dim=-1, descending=True).values
+    inf = torch.full((T,), float("inf"), dtype=z.dtype)
+    group_gap = best[:, keep - 1] - best[:, keep] if keep < groups else inf
+    kept = torch.topk(choice.view(T, groups, per).max(dim=-1).values, keep, dim=-1).indices
+    allowed = torch.zeros(T, groups, dtype=torch.bool)
+    allowed.scatter_(1, kept, True)
+    ranked = choice.masked_fill(~allowed.repeat_interleave(per, dim=1), float("-inf")).sort(dim=-1, descending=True).values
+    expert_gap = ranked[:, top - 1] - ranked[:, top] if top < keep * per else inf
+    return torch.minimum(group_gap, expert_gap)
+
+
 # --- the model --------------------------------------------------------------------
 
 class PlainMilenex:
@@ -134,9 +153,19 @@ class PlainMilenex:
                 self.w[name] = f.get_tensor(name).to(dtype)
         self.dtype = dtype
         self.eps = float(self.cfg["norm"]["eps"])
+        self.margins: List[torch.Tensor] = []      # of the last forward: every routed feed-forward run's route_margin
+
+    def closest_call(self) -> torch.Tensor:
+        """[T] of the last forward: per token the smallest routing margin of any layer run (infinite without routers)."""
+        return torch.stack(self.margins).min(dim=0).values if self.margins else None
 
     def lin(self, name: str, x: torch.Tensor) -> torch.Tensor:
         return x @ self.w[name].T
+
+    @staticmethod
+    def window(m: dict, T: int) -> int:
+        """The mixer's window; without one every earlier token is seen."""
+        return int(m["mask"]["size"]) if m.get("mask") is not None else T
 
     def attention(self, p: str, m: dict, h: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         T, H, G, d, e = h.shape[0], m["heads"], m["kv_heads"], m["dim"], m["vdim"]
@@ -152,13 +181,13 @@ class PlainMilenex:
         o = torch.zeros(T, H, e, dtype=h.dtype)
         for a in range(H):
             g = a // (H // G)
-            o[:, a] = window_weights(q[:, a], k[:, g], float(m["scale"]), int(m["mask"]["size"]), float(self.w[p + "sink"][a])) @ v[:, g]
+            o[:, a] = window_weights(q[:, a], k[:, g], float(m["scale"]), self.window(m, T), float(self.w[p + "sink"][a])) @ v[:, g]
         return self.lin(p + "o", o.reshape(T, H * e))
 
     def attention_2(self, p: str, m: dict, h: torch.Tensor) -> torch.Tensor:
         T, H, G, d, e = h.shape[0], m["heads"], m["kv_heads"], m["dim"], m["vdim"]
         q, k, v = self.lin(p + "q", h).view(T, H, d), self.lin(p + "k", h).view(T, G, d), self.lin(p + "v", h).view(T, G, e)
-        w = torch.stack([window_weights(q[:, a], k[:, a // (H // G)], float(m["scale"]), int(m["mask"]["size"]),
+        w = torch.stack([window_weights(q[:, a], k[:, a // (H // G)], float(m["scale"]), self.window(m, T),
                                         float(self.w[p + "sink"][a]), float(self.w[p + "r1"][a]), float(self.w[p + "r2"][a]))
                          for a in range(H)])
         mixed = torch.einsum("hg,gij->hij", self.w[p + "talk"], w)
@@ -175,8 +204,10 @@ class PlainMilenex:
         if m["kind"] == "dense":
             return self.lin(p + "down", gelu_erf(self.lin(p + "up", h)))
         r = m["router"]
-        chosen, weights = route(self.lin(p + "router", h), self.w[p + "correction"], int(r["top"]),
-                                int(r["groups"]["count"]), int(r["groups"]["keep"]))
+        groups = r.get("groups") or dict(count=1, keep=1)
+        z = self.lin(p + "router", h)
+        chosen, weights = route(z, self.w[p + "correction"], int(r["top"]), int(groups["count"]), int(groups["keep"]))
+        self.margins.append(route_margin(z, self.w[p + "correction"], int(r["top"]), int(groups["count"]), int(groups["keep"])))
         out = torch.zeros_like(h)
         for t in range(h.shape[0]):
             for e, wt in zip(chosen[t].tolist(), weights[t]):
@@ -215,6 +246,7 @@ class PlainMilenex:
         positions = torch.arange(len(ids))
         emb = self.w["embed"][ids]
         x = emb.clone()
+        self.margins = []
         after: List[torch.Tensor] = []
         for n, add in self.order():
             if add:
