@@ -12,6 +12,11 @@
 // mixes them and adds the values up.  A wave owns the heads w, w + waves, ...: their scores, their statistics, their
 // outputs.  Against keeping the scores of the first walk (heads x window floats a row) the second product costs less than
 // the memory would.  Caches: keys [page, kv_head, token, dim], values [page, kv_head, token, vdim].
+//
+// Few rows with long walks (decoding) would leave most of the GPU idle: then a row's keys are cut into parts, a workgroup
+// each, and the two walks become two launches -- the first leaves every part's maxima and sums, the second combines
+// them into the row's statistics, weighs its own part's values and leaves a partial output (the weights are finished,
+// so the parts' outputs simply add up) -- and a third adds the parts and applies the gate.
 #include <float.h>
 #include <math.h>
 
@@ -50,7 +55,10 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     const int32_t* __restrict__ positions, const float* __restrict__ sink, const float* __restrict__ far1,
     const float* __restrict__ far2, const float* __restrict__ talk, const void* __restrict__ gate, int gate_dtype,
     long gate_row, void* __restrict__ out, int out_dtype, int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens,
-    int window, float scale) {
+    int window, float scale, int n_parts, int phase, float* __restrict__ stats, float* __restrict__ partial) {
+  // phase 0: both walks over all keys, the finished output.  1: the first walk over this part's keys -> stats
+  // [row, part, head, (max, sum)].  2: the second walk over this part's keys with all parts' stats -> partial
+  // [row, part, head, vdim].
   extern __shared__ __align__(16) float dyn[];
   __shared__ long k_at[kMaxWaves][kWave];     // where every key of the tile lies (key/value head 0)
   __shared__ long v_at[kMaxWaves][kWave];
@@ -72,6 +80,14 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
 
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int total = pos - first + 1;
+  const int key_part = blockIdx.y;
+  int v_begin = 0, v_end = total;
+  if (n_parts > 1) {                          // whole tiles of 64 keys a part; the last parts may be empty
+    const int tiles = (total + kWave - 1) / kWave;
+    const int per = (tiles + n_parts - 1) / n_parts;
+    v_begin = key_part * per * kWave < total ? key_part * per * kWave : total;
+    v_end = v_begin + per * kWave < total ? v_begin + per * kWave : total;
+  }
   const bool by_four = dim % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
   const int sub = lane / 8, piece = lane % 8;
   int k_col[E4];
@@ -138,7 +154,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
   float mx[SL], inv[SL];
 #pragma unroll
   for (int s = 0; s < SL; ++s) mx[s] = -INFINITY, inv[s] = 0.f;
-  for (int v0 = 0; v0 < total; v0 += kWave) {
+  for (int v0 = v_begin; v0 < v_end && phase != 2; v0 += kWave) {
     bool seen;
     int j;
     place(v0, seen, j);
@@ -154,6 +170,31 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
       mx[s] = m_new;
     }
     wave_sync();
+  }
+  if (phase == 1) {                                         // this part's maxima and sums (an empty part: -inf, 0)
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const int h = wave + s * n_waves;
+      if (h >= n_heads) break;
+      float* at = stats + ((static_cast<long>(row) * n_parts + key_part) * n_heads + h) * 2;
+      if (lane == 0) at[0] = mx[s], at[1] = inv[s];
+    }
+    return;
+  }
+  if (phase == 2) {                                         // the row's statistics from every part's (the first is never empty)
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const int h = wave + s * n_waves;
+      if (h >= n_heads) break;
+      const float* of = stats + (static_cast<long>(row) * n_parts * n_heads + h) * 2;
+      float top = -INFINITY, sum = 0.f;
+      for (int i = 0; i < n_parts; ++i) top = fmaxf(top, of[static_cast<long>(i) * n_heads * 2]);
+      for (int i = 0; i < n_parts; ++i) {
+        const float m_i = of[static_cast<long>(i) * n_heads * 2];
+        if (m_i > -INFINITY) sum = fmaf(of[static_cast<long>(i) * n_heads * 2 + 1], expf(m_i - top), sum);
+      }
+      mx[s] = top, inv[s] = sum;
+    }
   }
 #pragma unroll
   for (int s = 0; s < SL; ++s) {
@@ -181,7 +222,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
   for (int s = 0; s < SL; ++s)
 #pragma unroll
     for (int i = 0; i < VPL; ++i) acc[s][i] = 0.f;
-  for (int v0 = 0; v0 < total; v0 += kWave) {
+  for (int v0 = v_begin; v0 < v_end; v0 += kWave) {
     bool seen;
     int j;
     place(v0, seen, j);
@@ -253,11 +294,35 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
       }
       const int c = vcol[i];
       if (c >= vdim || !writer) continue;
+      if (phase == 2) {
+        partial[((static_cast<long>(row) * n_parts + key_part) * n_heads + h) * vdim + c] = r;
+        continue;
+      }
       const long at = (static_cast<long>(row) * n_heads + h) * vdim + c;
       if (out_dtype == kF32) static_cast<float*>(out)[at] = r * g;
       else static_cast<bf16_t*>(out)[at] = from_float<bf16_t>(r * g);
     }
   }
+}
+
+// out[row, h, c] = sigmoid(gate[row, h]) * sum over the parts of partial[row, part, h, c].
+__global__ void attention_talk_finish_kernel(const float* __restrict__ partial, int n_parts, const void* __restrict__ gate,
+                                             int gate_dtype, long gate_row, void* __restrict__ out, int out_dtype, long n_rows,
+                                             int n_heads, int vdim) {
+  const long per_row = static_cast<long>(n_heads) * vdim;
+  const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n_rows * per_row) return;
+  const long row = i / per_row, rest = i % per_row;
+  const int h = static_cast<int>(rest / vdim);
+  float r = 0.f;
+  for (int p = 0; p < n_parts; ++p) r += partial[(row * n_parts + p) * per_row + rest];
+  if (gate) {
+    const long at = row * gate_row + h;
+    const float z = gate_dtype == kF32 ? static_cast<const float*>(gate)[at] : to_float(static_cast<const bf16_t*>(gate)[at]);
+    r *= 1.0f / (1.0f + expf(-z));
+  }
+  if (out_dtype == kF32) static_cast<float*>(out)[i] = r;
+  else static_cast<bf16_t*>(out)[i] = from_float<bf16_t>(r);
 }
 
 }  // namespace
@@ -270,7 +335,8 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
                                    const int32_t* positions, const float* sink, const float* far1, const float* far2,
                                    const float* talk, const void* gate, int gate_dtype, long gate_row, void* out,
                                    int out_dtype, int n_rows, int n_heads, int n_kv_heads, int dim, int vdim,
-                                   int page_tokens, int window, float scale, void* stream) {
+                                   int page_tokens, int window, float scale, int n_parts, float* stats, float* partial,
+                                   void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= kMaxHeads && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "attention_talk: bad sizes T=%d heads=%d/%d (at most %d heads)", n_rows, n_heads, n_kv_heads, kMaxHeads);
   BC4G_REQUIRE(dim > 0 && dim <= kMaxDim && vdim > 0 && vdim <= kMaxVdim, "attention_talk: dim=%d (at most %d), vdim=%d (at most %d)",
@@ -284,17 +350,21 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
                (!gate || gate_row >= n_heads) && (out_dtype == kF32 || out_dtype == kBF16) &&
                (!gate || gate_dtype == kF32 || gate_dtype == kBF16) && (far1 == nullptr) == (far2 == nullptr),
                "attention_talk: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
+  BC4G_REQUIRE(n_parts >= 1 && n_parts <= 65535 && (n_parts == 1 || (stats && partial)),
+               "attention_talk: %d parts of a row's keys need room for their statistics and outputs", n_parts);
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int waves = n_heads < kMaxWaves ? n_heads : kMaxWaves;
   const int slots = (n_heads + waves - 1) / waves;
   const size_t lds = static_cast<size_t>(n_heads) * (32 * e4 + kWave) * sizeof(float);
   const bool v_four = vdim % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
-#define BC4G_TALK(T, SL, E, V)                                                                                              \
-  attention_talk_kernel<T, SL, E, V><<<n_rows, waves * kWave, lds, s>>>(                                                    \
+#define BC4G_TALK_PHASE(T, SL, E, V, PHASE)                                                                                 \
+  attention_talk_kernel<T, SL, E, V><<<dim3(n_rows, n_parts), waves * kWave, lds, s>>>(                                     \
       q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table, table_stride, row_seq, positions, \
       sink, far1, far2, talk, gate, gate_dtype, gate_row, out, out_dtype, n_heads, n_kv_heads, dim, vdim, page_tokens, window, \
-      scale)
+      scale, n_parts, PHASE, stats, partial)
+#define BC4G_TALK(T, SL, E, V)                                                                                              \
+  do { if (n_parts == 1) BC4G_TALK_PHASE(T, SL, E, V, 0); else { BC4G_TALK_PHASE(T, SL, E, V, 1); BC4G_TALK_PHASE(T, SL, E, V, 2); } } while (0)
 #define BC4G_TALK_V(T, SL, E)                                                                                               \
   do { if (!v_four) BC4G_TALK(T, SL, E, 0); else if (vdim <= 64) BC4G_TALK(T, SL, E, 16); else if (vdim <= 128) BC4G_TALK(T, SL, E, 32); else BC4G_TALK(T, SL, E, 64); } while (0)
 #define BC4G_TALK_E(T, SL)                                                                                                  \
@@ -305,8 +375,14 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
   else if (cache_dtype == kBF16) BC4G_TALK_S(bf16_t);
   else return fail("attention_talk: unknown dtype %d", cache_dtype);
 #undef BC4G_TALK
+#undef BC4G_TALK_PHASE
 #undef BC4G_TALK_V
 #undef BC4G_TALK_E
 #undef BC4G_TALK_S
+  if (n_parts > 1) {
+    const long total = static_cast<long>(n_rows) * n_heads * vdim;
+    attention_talk_finish_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, s>>>(
+        partial, n_parts, gate, gate_dtype, gate_row, out, out_dtype, n_rows, n_heads, vdim);
+  }
   return check_launch("attention_talk");
 }

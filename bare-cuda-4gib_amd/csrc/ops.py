@@ -1723,6 +1723,8 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 TALK_MAX_HEADS = 64          # query heads whose weights attention_talk mixes
 TALK_MAX_QUERIES = 8192      # heads * (dim rounded up: 64 up to 64, else 256) that a row's queries may take in its LDS
+TALK_WORKGROUPS = 512        # a step of fewer rows cuts every row's keys into parts (whole tiles of 64) to bring this many
+TALK_MAX_PARTS = 64
 
 
 def attention_talk_takes(n_heads: int, dim: int, vdim: int) -> bool:
@@ -1733,13 +1735,15 @@ def attention_talk_takes(n_heads: int, dim: int, vdim: int) -> bool:
 def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
                    n_heads: int, n_kv_heads: int, dim: int, vdim: int, window: int, scale: float, *,
                    sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                   talk: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   talk: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, parts: int = 0) -> torch.Tensor:
     """Windowed softmax attention whose heads' weights are mixed before they meet the values: q float32 [T, n_heads, dim];
     keys [pages, n_kv_heads, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].  A row at position p sees key
     j <= p with p - j < window (0: every key).  score = q . k * scale - r1 ln(1 + r2 (p - j)) (``far`` = (r1, r2));
     w_g = exp(score_g) / (sum_j exp(score_g) + exp(sink_g)); head h weighs the values of its own key/value head by
     sum_g talk[h, g] w_g (``talk`` float32 [n_heads, n_heads]; none: its own weights) and is multiplied by
-    sigmoid(gate[t, h]) (``gate`` [T, n_heads], may be a part of wider rows).  Returns [T, n_heads * vdim]."""
+    sigmoid(gate[t, h]) (``gate`` [T, n_heads], may be a part of wider rows).  Returns [T, n_heads * vdim].
+    ``parts``: into how many parts, a workgroup each, every row's keys are cut (0: chosen here -- one where the rows fill
+    the GPU, more where few rows walk long contexts)."""
     _dev("attention_talk", q, k_cache, v_cache, block_table, sink, talk, *(far or ()))
     t = q.shape[0]
     if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, dim) or not q.is_contiguous():
@@ -1778,11 +1782,19 @@ def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         mixing = n_heads if talk is not None else 0
         return (2.0 * pairs * n_heads * (dim + vdim + mixing),
                 keys * n_kv_heads * (dim + vdim) * k_cache.element_size() + t * n_heads * (4 * dim + vdim * out.element_size()))
+    if parts <= 0:
+        reach = ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window)
+        parts = max(1, min(-(-reach // 64), TALK_MAX_PARTS, TALK_WORKGROUPS // max(1, t)))
+    stats = partial = None
+    if parts > 1:
+        stats = torch.empty((t, parts, n_heads, 2), dtype=torch.float32, device=q.device)
+        partial = torch.empty((t, parts, n_heads * vdim), dtype=torch.float32, device=q.device)
     library.call("bc4g_attention_talk", _ptr(q), n_heads * dim, _ptr(k_cache), _ptr(v_cache), _code(k_cache, "attention_talk"),
                  _ptr(block_table), block_table.stride(0), _ptr(ctx.row_seq), _ptr(ctx.positions), _ptr(sink),
                  _ptr(far[0]) if far else None, _ptr(far[1]) if far else None, _ptr(talk), _ptr(gate),
                  _code(gate, "attention_talk") if gate is not None else F32, gate_row, _ptr(out), _code(out, "attention_talk"),
-                 t, n_heads, n_kv_heads, dim, vdim, page_tokens, int(window), float(scale), _stream(), cost=cost)
+                 t, n_heads, n_kv_heads, dim, vdim, page_tokens, int(window), float(scale), int(parts), _ptr(stats), _ptr(partial),
+                 _stream(), cost=cost)
     return out
 
 

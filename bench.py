@@ -34,7 +34,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0                       # MI355X: 8 TB/s
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
-FP32_WORK = {"attention_maps", "decay_scan"}    # kernels whose arithmetic is float32 by their design's rule
+FP32_WORK = {"attention_maps", "attention_talk", "decay_scan"}    # kernels whose arithmetic is float32 by their design's rule
 TINYLLAMA = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=32000, hidden_size=2048,
                  num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
                  intermediate_size=5632, rope_theta=10000.0, rms_norm_eps=1e-5,
@@ -97,6 +97,31 @@ NAGEZEN_SIZES = {
     "1k": (nagezen_shape(1024, 6, 8, 2, 64, 128, 2752), MAMENEX_SIZES["1k"][0]),
     "2k": (nagezen_shape(2048, 6, 16, 4, 64, 128, 5504), MAMENEX_SIZES["2k"][0]),
     "4k": (nagezen_shape(4096, 6, 32, 8, 64, 128, 9600), MAMENEX_SIZES["4k"][0]),
+}
+
+
+def milenex_shape(width, layers, heads, kv_heads, dim, vdim, ff, experts, top, expert_ff, window=1024, vocab=32000):
+    """A Milenex configuration of real layer sizes: convolved, rotated sink attention and distance-penalised attention
+    with mixed heads in turn, all behind a token shift; the first layer's feed-forward dense, the others ``top`` of
+    ``experts`` routed experts in four groups of which three are kept, with a shared expert; the second layer runs twice."""
+    dense = dict(kind="dense", ff=ff)
+    moe = dict(kind="moe", expert=dict(ff=expert_ff, limit=7.0), router=dict(experts=experts, top=top, groups=dict(count=4, keep=3)),
+               shared=dict(ff=expert_ff, limit=7.0))
+    one = dict(type="attention", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, conv=4,
+                                            mask=dict(size=window), rot=dict(base=10000.0, dims=dim)))
+    two = dict(type="attention_2", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, mask=dict(size=window)))
+    order = [dict(one if i % 2 == 0 else two, mlp=dense if i == 0 else moe) for i in range(layers)]
+    return dict(architecture="Milenex", vocab=vocab, width=width, norm=dict(eps=1e-6), loop=dict(start=1, stop=2, times=2), layers=order)
+
+
+# --only milenex: the design at a few sizes that resemble a real model's layers (five layers, six layer runs; a row uses
+# two of eight experts and the shared one, together the parameters of the other design's feed-forward), each beside the
+# Nagezen decoder (the other design here with windowed attention in float32 heads and a clamped gated feed-forward) of
+# the same width, number of layer runs and head count.
+MILENEX_SIZES = {
+    "1k": (milenex_shape(1024, 5, 8, 2, 64, 128, 4096, 8, 2, 896), NAGEZEN_SIZES["1k"][0]),
+    "2k": (milenex_shape(2048, 5, 16, 4, 64, 128, 8192, 8, 2, 1792), NAGEZEN_SIZES["2k"][0]),
+    "4k": (milenex_shape(4096, 5, 32, 8, 64, 128, 14336, 8, 2, 3200), NAGEZEN_SIZES["4k"][0]),
 }
 BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
 
@@ -270,7 +295,7 @@ def kernel_table(model, cfg, prefill_tokens, batch, context, dtype):
 
 def run_mamenex(size, args, only="mamenex", names=("mamenex", "llama"), sizes=None):
     """Prefill and decode of a design at one size beside another decoder of equal size (Mamenex beside Llama, Nagezen
-    beside Mamenex); with --kernels the per-kernel tables of both."""
+    beside Mamenex, Milenex beside Nagezen); with --kernels the per-kernel tables of both."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     line = {"only": only, "size": size, "dtype": args.dtype, "prefill_tokens": args.prefill_tokens, "batch": args.batch,
@@ -438,9 +463,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
     ap.add_argument("--gather-ms", type=float, default=0.0,
                     help="--only chat: the scheduler waits this long before it admits those who came while others decode")
-    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex, --only nagezen: which of the sizes " + ", ".join(MAMENEX_SIZES))
-    ap.add_argument("--kernels", action="store_true", help="--only mamenex, --only nagezen: add the per-kernel tables (time, part of the roofline)")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex", "nagezen"], default=None,
+    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex, nagezen, milenex: which of the sizes " + ", ".join(MAMENEX_SIZES))
+    ap.add_argument("--kernels", action="store_true", help="--only mamenex, nagezen, milenex: add the per-kernel tables (time, part of the roofline)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex", "nagezen", "milenex"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
@@ -464,6 +489,10 @@ def main() -> int:
     if args.only == "nagezen":
         for size in args.sizes.split(","):
             print(json.dumps(run_mamenex(size, args, "nagezen", ("nagezen", "mamenex"), NAGEZEN_SIZES)), flush=True)
+        return 0
+    if args.only == "milenex":
+        for size in args.sizes.split(","):
+            print(json.dumps(run_mamenex(size, args, "milenex", ("milenex", "nagezen"), MILENEX_SIZES)), flush=True)
         return 0
     from bare_cuda_4gib_amd.csrc.peaks import measured_peaks
     measured = measured_peaks()

@@ -399,7 +399,7 @@ def plain_heads(q, keys, values, pos, G, scale, window, sink, far=None, talk=Non
     return out, weights
 
 
-def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk, gate):
+def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk, gate, parts=0):
     from bare_cuda_4gib_amd.csrc import ops
     dev = lambda t: t.to(DEV) if t is not None else None      # noqa: E731
     far = (dev(far[0].float()), dev(far[1].float())) if far is not None else None
@@ -409,7 +409,7 @@ def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, sc
                                   window, 0, scale, sink=dev(sink.float()), far=far).cpu().double()
     return ops.attention_talk(q_rows.contiguous().to(DEV), k_cache, v_cache, table, ctx, torch.float32, H, G, d, e, window, scale,
                               sink=dev(sink.float()), far=far, talk=dev(talk.float()) if talk is not None else None,
-                              gate=dev(gate)).cpu().double()
+                              gate=dev(gate), parts=parts).cpu().double()
 
 
 SIZES = [(4, 2, 12, 20), (3, 3, 10, 70), (6, 1, 44, 100), (2, 1, 7, 130), (2, 2, 72, 200), (12, 4, 6, 9), (18, 6, 8, 12)]
@@ -450,6 +450,35 @@ def test_attention_finds_one_key_among_hundreds(dtype, kind, needle, sizes):
             assert torch.allclose(got[r].view(H, e), want, atol=tol * max(1.0, float(want.abs().max())), rtol=tol), (needle, pos)
             if needle <= pos:
                 assert float(weights[mark][needle]) > 0.9
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("parts", [1, 2, 3, 5, 64])
+@pytest.mark.parametrize("window", [0, 100, 64])
+def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window):
+    """The keys of every row cut into one to 64 parts (more parts than tiles of keys: the last are empty), a needle in the
+    last part's tile, rows of unequal reach in one step: the parts' statistics and outputs add up to the plain result."""
+    torch.manual_seed(parts)
+    H, G, d, e, n, P, scale = 6, 2, 24, 36, 300, 16, 0.3
+    keys, values = (torch.randn(n, G, d) * 0.3).to(dtype).float(), torch.randn(n, G, e).to(dtype).float()
+    q = torch.randn(H, d)
+    sink, far = torch.randn(H) + 1.0, (torch.rand(H) * 0.5 + 0.2, torch.rand(H) * 2.0 + 0.1)
+    talk = torch.eye(H) * 0.8 + torch.randn(H, H) * 0.25
+    keys[n - 3, 1] = (q[4] / float(q[4] @ q[4]) * 20.0 / scale).to(dtype).float()
+    pages = torch.randperm(30)[:-(-n // P)]
+    k_cache, v_cache = paged(keys, values, pages, P, dtype, 30)
+    table = pages.to(torch.int32).view(1, -1).repeat(2, 1).to(DEV)         # two requests over the same pages
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    lengths, cached = [3, 1], [n - 3, 40]
+    ctx = step_context(lengths, cached, [0, 1])
+    gate = torch.randn(4, H)
+    got = run_heads("mixed", q.view(1, H, d).repeat(4, 1, 1), k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk,
+                    gate, parts=parts)
+    for r, pos in enumerate([n - 3, n - 2, n - 1, 40]):
+        want, weights = plain_heads(q, keys, values, pos, G, scale, window, sink, far, talk, gate[r])
+        assert torch.allclose(got[r].view(H, e), want, atol=tol * max(1.0, float(want.abs().max())), rtol=tol), (parts, pos)
+        if pos >= n - 3:
+            assert float(weights[4][n - 3]) > 0.9
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
