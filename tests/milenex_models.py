@@ -72,8 +72,15 @@ CONFIGS: Dict[str, dict] = {
         attention(2, 2, 8, 8, mlp=dense(48)),                                      # no window, no convolution, no rotation
         attention(4, 4, 4, 3, window=64, conv=2, dims=2, base=7.0, scale=1.1, mlp=None),
         attention_2(18, 6, 8, 12, window=65, scale=0.5, mlp=moe(3, 2, 16, 1.0, groups=(1, 1), shared=(8, 1.0)))]),
+    # ones and equals: a window of one key (the row's own) and of two, one tap, one head, one expert a group with every group
+    # kept, one expert in all, a loop over every layer, a rotation of one pair
+    "E": dict(architecture="Milenex", vocab=50, width=24, norm=dict(eps=1e-6), loop=dict(start=0, stop=4, times=2), layers=[
+        attention_2(1, 1, 4, 4, window=1, scale=1.0, mlp=moe(4, 1, 8, 2.0, groups=(4, 4))),
+        attention(1, 1, 2, 1, window=2, conv=1, dims=2, base=2.0, scale=1.0, mlp=moe(1, 1, 8, 1.0, shared=(8, 1.0))),
+        attention_2(4, 4, 4, 4, window=128, mlp=dense(8)),
+        attention(3, 3, 6, 2, window=1, conv=2, dims=4, mlp=moe(6, 2, 8, 1.0, groups=(6, 2)))]),
 }
-SEEDS = {"A": 13, "B": 24, "C": 35, "D": 46}
+SEEDS = {"A": 13, "B": 24, "C": 35, "D": 46, "E": 57}
 
 
 def every_expert(config: dict) -> dict:

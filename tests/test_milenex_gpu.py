@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 # A row of logits may differ from the plain row by this fraction of the plain row's root mean square (the errors' root
 # mean square over the vocabulary), and no single logit by more than ten times that.
 ROW_RMS = {"float32": 2e-5, "bfloat16": 6e-2}
-LENGTHS = {"A": [1, 2, 9, 70, 150], "B": [3, 33, 64, 129], "C": [1, 17, 140], "D": [2, 66, 131, 200]}
+LENGTHS = {"A": [1, 2, 9, 70, 150], "B": [3, 33, 64, 129], "C": [1, 17, 140], "D": [2, 66, 131, 200], "E": [1, 2, 3, 65, 190]}
 CLOSE_CALL = 1e-5       # a 32-bit run is held to the plain rows up to a request's first routing margin below this
 
 
