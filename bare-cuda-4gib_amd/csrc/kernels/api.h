@@ -353,12 +353,14 @@ int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const v
 // if a gate [T, heads] is given (rows gate_row apart).  sink, far1/far2 and talk ([heads, heads]) may each be null.
 // heads * dim at most 8192, heads at most 64.  n_parts > 1: every row's keys are cut into that many parts, a workgroup each;
 // stats (float [T, n_parts, heads, 2]) and partial (float [T, n_parts, heads, vdim]) are the room they need.
+// kept (float [T, heads, kept_stride], kept_stride whole tiles of 64 that hold a row's visible keys; may be null): room for
+// the first walk's scores, which the second walk then reads instead of computing them again.
 int bc4g_attention_talk(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
                         const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                         const float* sink, const float* far1, const float* far2, const float* talk, const void* gate,
                         int gate_dtype, long gate_row, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads,
                         int dim, int vdim, int page_tokens, int window, float scale, int n_parts, float* stats, float* partial,
-                        void* stream);
+                        float* kept, long kept_stride, void* stream);
 
 // out[t, :] += float(table[ids[t], :]): the embedding once more, added to the stream.
 int bc4g_embed_add(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden, int vocab,

@@ -10,8 +10,10 @@
 // known: so a workgroup is one row with all its heads, and it walks the row's keys twice.  The first walk leaves every
 // head's maximum and denominator; the second works the scores out again, turns them into weights in LDS (head x 64 keys),
 // mixes them and adds the values up.  A wave owns the heads w, w + waves, ...: their scores, their statistics, their
-// outputs.  Against keeping the scores of the first walk (heads x window floats a row) the second product costs less than
-// the memory would.  Caches: keys [page, kv_head, token, dim], values [page, kv_head, token, vdim].
+// outputs.  Where the caller gives room for them (heads x reach floats a row, in memory: LDS could not hold them), the
+// first walk leaves its scores there and the second reads them back -- a lane reads what it wrote itself -- instead of
+// working the products out again; without that room the second walk computes them once more.
+// Caches: keys [page, kv_head, token, dim], values [page, kv_head, token, vdim].
 //
 // Few rows with long walks (decoding) would leave most of the GPU idle: then a row's keys are cut into parts, a workgroup
 // each, and the two walks become two launches -- the first leaves every part's maxima and sums, the second combines
@@ -55,10 +57,11 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     const int32_t* __restrict__ positions, const float* __restrict__ sink, const float* __restrict__ far1,
     const float* __restrict__ far2, const float* __restrict__ talk, const void* __restrict__ gate, int gate_dtype,
     long gate_row, void* __restrict__ out, int out_dtype, int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens,
-    int window, float scale, int n_parts, int phase, float* __restrict__ stats, float* __restrict__ partial) {
+    int window, float scale, int n_parts, int phase, float* __restrict__ stats, float* __restrict__ partial,
+    float* __restrict__ kept, long kept_stride) {
   // phase 0: both walks over all keys, the finished output.  1: the first walk over this part's keys -> stats
   // [row, part, head, (max, sum)].  2: the second walk over this part's keys with all parts' stats -> partial
-  // [row, part, head, vdim].
+  // [row, part, head, vdim].  kept [row, head, kept_stride]: the first walk's scores, by visible key (or null).
   extern __shared__ __align__(16) float dyn[];
   __shared__ long k_at[kMaxWaves][kWave];     // where every key of the tile lies (key/value head 0)
   __shared__ long v_at[kMaxWaves][kWave];
@@ -163,6 +166,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
       float sc = scores(h, j);
+      if (kept) kept[(static_cast<long>(row) * n_heads + h) * kept_stride + v0 + lane] = sc;
       if (!seen) sc = -INFINITY;
       const float m_new = fmaxf(mx[s], wave_max(sc));       // finite: the tile's first key is visible
       const float p = seen ? expf(sc - m_new) : 0.f;
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     for (int s = 0; s < SL; ++s) {
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
-      const float sc = scores(h, j);
+      const float sc = kept ? kept[(static_cast<long>(row) * n_heads + h) * kept_stride + v0 + lane] : scores(h, j);
       p_s[h * kWave + lane] = seen ? expf(sc - mx[s]) * inv[s] : 0.f;
     }
     __syncthreads();                                        // every head's weights of this tile are there
@@ -336,7 +340,7 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
                                    const float* talk, const void* gate, int gate_dtype, long gate_row, void* out,
                                    int out_dtype, int n_rows, int n_heads, int n_kv_heads, int dim, int vdim,
                                    int page_tokens, int window, float scale, int n_parts, float* stats, float* partial,
-                                   void* stream) {
+                                   float* kept, long kept_stride, void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= kMaxHeads && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "attention_talk: bad sizes T=%d heads=%d/%d (at most %d heads)", n_rows, n_heads, n_kv_heads, kMaxHeads);
   BC4G_REQUIRE(dim > 0 && dim <= kMaxDim && vdim > 0 && vdim <= kMaxVdim, "attention_talk: dim=%d (at most %d), vdim=%d (at most %d)",
@@ -352,6 +356,8 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
                "attention_talk: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
   BC4G_REQUIRE(n_parts >= 1 && n_parts <= 65535 && (n_parts == 1 || (stats && partial)),
                "attention_talk: %d parts of a row's keys need room for their statistics and outputs", n_parts);
+  BC4G_REQUIRE(!kept || (kept_stride > 0 && kept_stride % kWave == 0), "attention_talk: the kept scores' rows (%ld) must be whole tiles of %d",
+               kept_stride, kWave);
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int waves = n_heads < kMaxWaves ? n_heads : kMaxWaves;
@@ -362,7 +368,7 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
   attention_talk_kernel<T, SL, E, V><<<dim3(n_rows, n_parts), waves * kWave, lds, s>>>(                                     \
       q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table, table_stride, row_seq, positions, \
       sink, far1, far2, talk, gate, gate_dtype, gate_row, out, out_dtype, n_heads, n_kv_heads, dim, vdim, page_tokens, window, \
-      scale, n_parts, PHASE, stats, partial)
+      scale, n_parts, PHASE, stats, partial, kept, kept_stride)
 #define BC4G_TALK(T, SL, E, V)                                                                                              \
   do { if (n_parts == 1) BC4G_TALK_PHASE(T, SL, E, V, 0); else { BC4G_TALK_PHASE(T, SL, E, V, 1); BC4G_TALK_PHASE(T, SL, E, V, 2); } } while (0)
 #define BC4G_TALK_V(T, SL, E)                                                                                               \

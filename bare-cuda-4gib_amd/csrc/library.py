@@ -63,7 +63,7 @@ _SIGNATURES = {
     "bc4g_attention_maps": [_P, c_long, _P, _P, _I, _P, _I, _P, _P, _F, _I, _F, _F, _P, _I, c_long, _I, _P, _I,
                             _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, _P],
     "bc4g_attention_talk": [_P, c_long, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, c_long, _P, _I,
-                            _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
+                            _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, c_long, _P],
     "bc4g_embed_add": [_P, _I, _P, _P, _I, _I, _I, _P],
     "bc4g_gelu": [_P, _P, _I, c_long, _P],
     "bc4g_moe_route": [_P, c_long, _P, _P, _P, _I, _I, _I, _I, _I, _P],

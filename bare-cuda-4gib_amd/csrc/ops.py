@@ -1725,6 +1725,7 @@ TALK_MAX_HEADS = 64          # query heads whose weights attention_talk mixes
 TALK_MAX_QUERIES = 8192      # heads * (dim rounded up: 64 up to 64, else 256) that a row's queries may take in its LDS
 TALK_WORKGROUPS = 512        # a step of fewer rows cuts every row's keys into parts (whole tiles of 64) to bring this many
 TALK_MAX_PARTS = 64
+TALK_KEPT_BYTES = 1 << 30    # the most a step's first-walk scores may take to be kept for the second walk (else: computed twice)
 
 
 def attention_talk_takes(n_heads: int, dim: int, vdim: int) -> bool:
@@ -1735,7 +1736,8 @@ def attention_talk_takes(n_heads: int, dim: int, vdim: int) -> bool:
 def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, ctx, out_dtype: torch.dtype,
                    n_heads: int, n_kv_heads: int, dim: int, vdim: int, window: int, scale: float, *,
                    sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                   talk: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, parts: int = 0) -> torch.Tensor:
+                   talk: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, parts: int = 0,
+                   keep_scores: Optional[bool] = None) -> torch.Tensor:
     """Windowed softmax attention whose heads' weights are mixed before they meet the values: q float32 [T, n_heads, dim];
     keys [pages, n_kv_heads, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].  A row at position p sees key
     j <= p with p - j < window (0: every key).  score = q . k * scale - r1 ln(1 + r2 (p - j)) (``far`` = (r1, r2));
@@ -1743,7 +1745,8 @@ def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     sum_g talk[h, g] w_g (``talk`` float32 [n_heads, n_heads]; none: its own weights) and is multiplied by
     sigmoid(gate[t, h]) (``gate`` [T, n_heads], may be a part of wider rows).  Returns [T, n_heads * vdim].
     ``parts``: into how many parts, a workgroup each, every row's keys are cut (0: chosen here -- one where the rows fill
-    the GPU, more where few rows walk long contexts)."""
+    the GPU, more where few rows walk long contexts).  ``keep_scores``: whether the first walk's scores are kept in memory
+    for the second (None: where they fit TALK_KEPT_BYTES)."""
     _dev("attention_talk", q, k_cache, v_cache, block_table, sink, talk, *(far or ()))
     t = q.shape[0]
     if q.dtype != torch.float32 or tuple(q.shape) != (t, n_heads, dim) or not q.is_contiguous():
@@ -1785,6 +1788,11 @@ def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if parts <= 0:
         reach = ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window)
         parts = max(1, min(-(-reach // 64), TALK_MAX_PARTS, TALK_WORKGROUPS // max(1, t)))
+    reach = ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window)
+    kept_row = 64 * max(1, -(-reach // 64))
+    if keep_scores is None:
+        keep_scores = 4 * t * n_heads * kept_row <= TALK_KEPT_BYTES
+    kept = torch.empty((t, n_heads, kept_row), dtype=torch.float32, device=q.device) if keep_scores else None
     stats = partial = None
     if parts > 1:
         stats = torch.empty((t, parts, n_heads, 2), dtype=torch.float32, device=q.device)
@@ -1794,7 +1802,7 @@ def attention_talk(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                  _ptr(far[0]) if far else None, _ptr(far[1]) if far else None, _ptr(talk), _ptr(gate),
                  _code(gate, "attention_talk") if gate is not None else F32, gate_row, _ptr(out), _code(out, "attention_talk"),
                  t, n_heads, n_kv_heads, dim, vdim, page_tokens, int(window), float(scale), int(parts), _ptr(stats), _ptr(partial),
-                 _stream(), cost=cost)
+                 _ptr(kept), kept_row, _stream(), cost=cost)
     return out
 
 

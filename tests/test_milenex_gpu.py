@@ -399,7 +399,7 @@ def plain_heads(q, keys, values, pos, G, scale, window, sink, far=None, talk=Non
     return out, weights
 
 
-def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk, gate, parts=0):
+def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk, gate, parts=0, keep=None):
     from bare_cuda_4gib_amd.csrc import ops
     dev = lambda t: t.to(DEV) if t is not None else None      # noqa: E731
     far = (dev(far[0].float()), dev(far[1].float())) if far is not None else None
@@ -409,7 +409,7 @@ def run_heads(kind, q_rows, k_cache, v_cache, table, ctx, H, G, d, e, window, sc
                                   window, 0, scale, sink=dev(sink.float()), far=far).cpu().double()
     return ops.attention_talk(q_rows.contiguous().to(DEV), k_cache, v_cache, table, ctx, torch.float32, H, G, d, e, window, scale,
                               sink=dev(sink.float()), far=far, talk=dev(talk.float()) if talk is not None else None,
-                              gate=dev(gate), parts=parts).cpu().double()
+                              gate=dev(gate), parts=parts, keep_scores=keep).cpu().double()
 
 
 SIZES = [(4, 2, 12, 20), (3, 3, 10, 70), (6, 1, 44, 100), (2, 1, 7, 130), (2, 2, 72, 200), (12, 4, 6, 9), (18, 6, 8, 12)]
@@ -455,9 +455,11 @@ def test_attention_finds_one_key_among_hundreds(dtype, kind, needle, sizes):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("parts", [1, 2, 3, 5, 64])
 @pytest.mark.parametrize("window", [0, 100, 64])
-def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window):
+@pytest.mark.parametrize("keep", [True, False])
+def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window, keep):
     """The keys of every row cut into one to 64 parts (more parts than tiles of keys: the last are empty), a needle in the
-    last part's tile, rows of unequal reach in one step: the parts' statistics and outputs add up to the plain result."""
+    last part's tile, rows of unequal reach in one step: the parts' statistics and outputs add up to the plain result,
+    with the first walk's scores kept for the second and without."""
     torch.manual_seed(parts)
     H, G, d, e, n, P, scale = 6, 2, 24, 36, 300, 16, 0.3
     keys, values = (torch.randn(n, G, d) * 0.3).to(dtype).float(), torch.randn(n, G, e).to(dtype).float()
@@ -473,7 +475,7 @@ def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window):
     ctx = step_context(lengths, cached, [0, 1])
     gate = torch.randn(4, H)
     got = run_heads("mixed", q.view(1, H, d).repeat(4, 1, 1), k_cache, v_cache, table, ctx, H, G, d, e, window, scale, sink, far, talk,
-                    gate, parts=parts)
+                    gate, parts=parts, keep=keep)
     for r, pos in enumerate([n - 3, n - 2, n - 1, 40]):
         want, weights = plain_heads(q, keys, values, pos, G, scale, window, sink, far, talk, gate[r])
         assert torch.allclose(got[r].view(H, e), want, atol=tol * max(1.0, float(want.abs().max())), rtol=tol), (parts, pos)
