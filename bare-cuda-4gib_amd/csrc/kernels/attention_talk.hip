@@ -18,7 +18,10 @@
 // Few rows with long walks (decoding) would leave most of the GPU idle: then a row's keys are cut into parts, a workgroup
 // each, and the two walks become two launches -- the first leaves every part's maxima and sums, the second combines
 // them into the row's statistics, weighs its own part's values and leaves a partial output (the weights are finished,
-// so the parts' outputs simply add up) -- and a third adds the parts and applies the gate.
+// so the parts' outputs simply add up) -- and a third adds the parts and applies the gate.  With kept scores the cut
+// goes on through the heads: workgroup z of a part takes the z-th head of every wave (its scores and statistics in
+// the first launch, its mixing and its weighted sums in the second, where every head's weights of the tile are made
+// from the kept scores by whoever needs them).
 #include <float.h>
 #include <math.h>
 
@@ -58,7 +61,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     const float* __restrict__ far2, const float* __restrict__ talk, const void* __restrict__ gate, int gate_dtype,
     long gate_row, void* __restrict__ out, int out_dtype, int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens,
     int window, float scale, int n_parts, int phase, float* __restrict__ stats, float* __restrict__ partial,
-    float* __restrict__ kept, long kept_stride) {
+    float* __restrict__ kept, long kept_stride, int by_slot) {
   // phase 0: both walks over all keys, the finished output.  1: the first walk over this part's keys -> stats
   // [row, part, head, (max, sum)].  2: the second walk over this part's keys with all parts' stats -> partial
   // [row, part, head, vdim].  kept [row, head, kept_stride]: the first walk's scores, by visible key (or null).
@@ -84,6 +87,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int total = pos - first + 1;
   const int key_part = blockIdx.y;
+  const int only = by_slot ? static_cast<int>(blockIdx.z) : -1;      // the one head of each wave this workgroup serves (-1: all)
   int v_begin = 0, v_end = total;
   if (n_parts > 1) {                          // whole tiles of 64 keys a part; the last parts may be empty
     const int tiles = (total + kWave - 1) / kWave;
@@ -165,6 +169,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     for (int s = 0; s < SL; ++s) {
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
+      if (only >= 0 && s != only) continue;
       float sc = scores(h, j);
       if (kept) kept[(static_cast<long>(row) * n_heads + h) * kept_stride + v0 + lane] = sc;
       if (!seen) sc = -INFINITY;
@@ -180,6 +185,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     for (int s = 0; s < SL; ++s) {
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
+      if (only >= 0 && s != only) continue;
       float* at = stats + ((static_cast<long>(row) * n_parts + key_part) * n_heads + h) * 2;
       if (lane == 0) at[0] = mx[s], at[1] = inv[s];
     }
@@ -191,12 +197,11 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
       const float* of = stats + (static_cast<long>(row) * n_parts * n_heads + h) * 2;
-      float top = -INFINITY, sum = 0.f;
-      for (int i = 0; i < n_parts; ++i) top = fmaxf(top, of[static_cast<long>(i) * n_heads * 2]);
-      for (int i = 0; i < n_parts; ++i) {
-        const float m_i = of[static_cast<long>(i) * n_heads * 2];
-        if (m_i > -INFINITY) sum = fmaf(of[static_cast<long>(i) * n_heads * 2 + 1], expf(m_i - top), sum);
-      }
+      const bool mine = lane < n_parts;                     // a lane a part (at most 64): one trip to memory for all of them
+      const float m_i = mine ? of[static_cast<long>(lane) * n_heads * 2] : -INFINITY;
+      const float s_i = mine ? of[static_cast<long>(lane) * n_heads * 2 + 1] : 0.f;
+      const float top = wave_max(m_i);
+      const float sum = wave_sum(m_i > -INFINITY ? s_i * expf(m_i - top) : 0.f);
       mx[s] = top, inv[s] = sum;
     }
   }
@@ -243,6 +248,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     for (int s = 0; s < SL; ++s) {
       const int h = wave + s * n_waves;
       if (h >= n_heads) break;
+      if (only >= 0 && s != only) continue;
       float mixed;
       if (talk) {
         mixed = 0.f;
@@ -283,6 +289,7 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
   for (int s = 0; s < SL; ++s) {
     const int h = wave + s * n_waves;
     if (h >= n_heads) break;
+    if (only >= 0 && s != only) continue;
     float g = 1.0f;
     if (gate) {
       const long at = row * gate_row + h;
@@ -354,7 +361,7 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
                (!gate || gate_row >= n_heads) && (out_dtype == kF32 || out_dtype == kBF16) &&
                (!gate || gate_dtype == kF32 || gate_dtype == kBF16) && (far1 == nullptr) == (far2 == nullptr),
                "attention_talk: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
-  BC4G_REQUIRE(n_parts >= 1 && n_parts <= 65535 && (n_parts == 1 || (stats && partial)),
+  BC4G_REQUIRE(n_parts >= 1 && n_parts <= kWave && (n_parts == 1 || (stats && partial)),
                "attention_talk: %d parts of a row's keys need room for their statistics and outputs", n_parts);
   BC4G_REQUIRE(!kept || (kept_stride > 0 && kept_stride % kWave == 0), "attention_talk: the kept scores' rows (%ld) must be whole tiles of %d",
                kept_stride, kWave);
@@ -362,13 +369,14 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int waves = n_heads < kMaxWaves ? n_heads : kMaxWaves;
   const int slots = (n_heads + waves - 1) / waves;
+  const int by_slot = n_parts > 1 && kept && slots > 1;
   const size_t lds = static_cast<size_t>(n_heads) * (32 * e4 + kWave) * sizeof(float);
   const bool v_four = vdim % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
 #define BC4G_TALK_PHASE(T, SL, E, V, PHASE)                                                                                 \
-  attention_talk_kernel<T, SL, E, V><<<dim3(n_rows, n_parts), waves * kWave, lds, s>>>(                                     \
+  attention_talk_kernel<T, SL, E, V><<<dim3(n_rows, n_parts, by_slot ? slots : 1), waves * kWave, lds, s>>>(                \
       q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), block_table, table_stride, row_seq, positions, \
       sink, far1, far2, talk, gate, gate_dtype, gate_row, out, out_dtype, n_heads, n_kv_heads, dim, vdim, page_tokens, window, \
-      scale, n_parts, PHASE, stats, partial, kept, kept_stride)
+      scale, n_parts, PHASE, stats, partial, kept, kept_stride, by_slot)
 #define BC4G_TALK(T, SL, E, V)                                                                                              \
   do { if (n_parts == 1) BC4G_TALK_PHASE(T, SL, E, V, 0); else { BC4G_TALK_PHASE(T, SL, E, V, 1); BC4G_TALK_PHASE(T, SL, E, V, 2); } } while (0)
 #define BC4G_TALK_V(T, SL, E)                                                                                               \

@@ -456,17 +456,19 @@ def test_attention_finds_one_key_among_hundreds(dtype, kind, needle, sizes):
 @pytest.mark.parametrize("parts", [1, 2, 3, 5, 64])
 @pytest.mark.parametrize("window", [0, 100, 64])
 @pytest.mark.parametrize("keep", [True, False])
-def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window, keep):
+@pytest.mark.parametrize("H,G", [(6, 2), (18, 6), (20, 1)])
+def test_mixed_heads_with_a_row_s_keys_cut_into_parts(dtype, parts, window, keep, H, G):
     """The keys of every row cut into one to 64 parts (more parts than tiles of keys: the last are empty), a needle in the
     last part's tile, rows of unequal reach in one step: the parts' statistics and outputs add up to the plain result,
-    with the first walk's scores kept for the second and without."""
+    with the first walk's scores kept for the second and without; with more heads than a workgroup has waves the kept
+    scores let the heads be cut over workgroups too."""
     torch.manual_seed(parts)
-    H, G, d, e, n, P, scale = 6, 2, 24, 36, 300, 16, 0.3
+    d, e, n, P, scale = 24, 36, 300, 16, 0.3
     keys, values = (torch.randn(n, G, d) * 0.3).to(dtype).float(), torch.randn(n, G, e).to(dtype).float()
     q = torch.randn(H, d)
     sink, far = torch.randn(H) + 1.0, (torch.rand(H) * 0.5 + 0.2, torch.rand(H) * 2.0 + 0.1)
     talk = torch.eye(H) * 0.8 + torch.randn(H, H) * 0.25
-    keys[n - 3, 1] = (q[4] / float(q[4] @ q[4]) * 20.0 / scale).to(dtype).float()
+    keys[n - 3, 4 // (H // G)] = (q[4] / float(q[4] @ q[4]) * 20.0 / scale).to(dtype).float()
     pages = torch.randperm(30)[:-(-n // P)]
     k_cache, v_cache = paged(keys, values, pages, P, dtype, 30)
     table = pages.to(torch.int32).view(1, -1).repeat(2, 1).to(DEV)         # two requests over the same pages
