@@ -228,6 +228,14 @@ int bc4g_rmsnorm_add(float* x, const void* y, int y_dtype, const float* w, int n
 // otherwise; pq = (p, q) float32 on the device.
 int bc4g_xielu(const void* in, void* out, int dtype, const float* pq, long total, void* stream);
 
+// out[t] = h[t] + (h[t - 1] - h[t]) * mix, h = x * rsqrt(mean(x^2) + eps) * w rounded to ``dtype`` (out's and state's): an RMS
+// norm of the float32 stream and the token shift behind it.  h[-1] of a request's first row of the step is its state
+// [slots, hidden] (zero when the request was admitted), which then receives the h of the request's last row.  The step's
+// rows are grouped by request: row_seq [T], seq_start [S + 1], seq_slots [S].  w, mix: float32 [hidden].
+int bc4g_rmsnorm_shift(const float* x, const float* w, const float* mix, void* out, void* state, int dtype,
+                       const int32_t* row_seq, const int32_t* seq_start, const int32_t* seq_slots, int n_rows, int hidden,
+                       float eps, void* stream);
+
 // A causal convolution over time on each channel, across steps: out[t, c] = (add_input ? in[t, c] : 0) + out_bias[c] +
 // sum_j w[j, c] * input(t - taps + 1 + j)[c] (w comes by taps, [taps][channels], so that neighbouring channels lie side
 // by side; its last row is the current token's), where a row's input is in[row] + in_bias (rounded to the storage type) and

@@ -114,6 +114,83 @@ int grid_for(long total) {
   return static_cast<int>(g < 1 ? 1 : (g > 65535 ? 65535 : g));
 }
 
+// out[t] = h[t] + (h[t - 1] - h[t]) * mix with h = (x * rsqrt(mean(x^2) + eps) * w rounded to the output's type): an RMS
+// norm and the token shift behind it in one pass.  A workgroup is one row; it works out the row before once more from
+// the stream (that row is in the cache) instead of waiting for it.  A request's first row of the step reads its state
+// (the h of its last row so far; zeros when it was admitted), and the same workgroup -- so nobody reads what another
+// writes -- leaves the h of the request's last row of this step there.  V elements a thread and trip (4 where the width
+// and the addresses allow: 16-byte loads, all of a pass in flight together).
+template <int V> struct Pack { float v[V]; };
+template <int V> __device__ inline Pack<V> load_pack(const float* p) {
+  Pack<V> r;
+  if (V == 4) { const float4 f = *reinterpret_cast<const float4*>(p); r.v[0] = f.x, r.v[1 % V] = f.y, r.v[2 % V] = f.z, r.v[3 % V] = f.w; }
+  else r.v[0] = p[0];
+  return r;
+}
+template <int V> __device__ inline Pack<V> load_pack(const bf16_t* p) {
+  Pack<V> r;
+  if (V == 4) {
+    const uint2 b = *reinterpret_cast<const uint2*>(p);
+    r.v[0] = __uint_as_float(b.x << 16), r.v[1 % V] = __uint_as_float(b.x & 0xffff0000u);
+    r.v[2 % V] = __uint_as_float(b.y << 16), r.v[3 % V] = __uint_as_float(b.y & 0xffff0000u);
+  } else r.v[0] = to_float(p[0]);
+  return r;
+}
+template <int V> __device__ inline void store_pack(float* p, const Pack<V>& r) {
+  if (V == 4) *reinterpret_cast<float4*>(p) = make_float4(r.v[0], r.v[1 % V], r.v[2 % V], r.v[3 % V]);
+  else p[0] = r.v[0];
+}
+template <int V> __device__ inline void store_pack(bf16_t* p, const Pack<V>& r) {
+  if (V == 4) {
+    uint2 b;
+    b.x = bf16_bits_from_float(r.v[0]) | (static_cast<uint32_t>(bf16_bits_from_float(r.v[1 % V])) << 16);
+    b.y = bf16_bits_from_float(r.v[2 % V]) | (static_cast<uint32_t>(bf16_bits_from_float(r.v[3 % V])) << 16);
+    *reinterpret_cast<uint2*>(p) = b;
+  } else p[0] = from_float<bf16_t>(r.v[0]);
+}
+
+template <typename TO, int V>
+__global__ __launch_bounds__(kBlock) void rmsnorm_shift_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                               const float* __restrict__ mix, TO* __restrict__ out,
+                                                               TO* __restrict__ state, const int32_t* __restrict__ row_seq,
+                                                               const int32_t* __restrict__ seq_start,
+                                                               const int32_t* __restrict__ seq_slots, int hidden, float eps) {
+  __shared__ float scratch[3][16];
+  const int row = blockIdx.x, seq = row_seq[row];
+  const int first = seq_start[seq], last = seq_start[seq + 1] - 1;
+  const bool from_state = row == first;                     // (the same for every thread of the workgroup)
+  const float* xr = x + static_cast<size_t>(row) * hidden;
+  const float* xo = from_state ? x + static_cast<size_t>(last) * hidden : xr - hidden;   // the other row this workgroup norms
+  const bool other = !from_state || last != row;
+  float ss = 0.f, so = 0.f;
+#pragma unroll 4
+  for (int i = V * threadIdx.x; i < hidden; i += V * kBlock) {
+    const Pack<V> a = load_pack<V>(xr + i), b = other ? load_pack<V>(xo + i) : a;
+#pragma unroll
+    for (int e = 0; e < V; ++e) ss = fmaf(a.v[e], a.v[e], ss), so = fmaf(b.v[e], b.v[e], so);
+  }
+  const float rs = 1.0f / sqrtf(block_sum(ss, scratch[0]) / static_cast<float>(hidden) + eps);
+  const float ro = 1.0f / sqrtf(block_sum(so, scratch[1]) / static_cast<float>(hidden) + eps);
+  TO* st = state + static_cast<size_t>(seq_slots[seq]) * hidden;
+  TO* orow = out + static_cast<size_t>(row) * hidden;
+#pragma unroll 4
+  for (int i = V * threadIdx.x; i < hidden; i += V * kBlock) {
+    const Pack<V> a = load_pack<V>(xr + i), b = other ? load_pack<V>(xo + i) : a, wi = load_pack<V>(w + i), mi = load_pack<V>(mix + i);
+    Pack<V> before, h, o, keep;
+    if (from_state) before = load_pack<V>(st + i);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      h.v[e] = to_float(from_float<TO>(a.v[e] * rs * wi.v[e]));
+      const float ho = to_float(from_float<TO>(b.v[e] * ro * wi.v[e]));      // the row before, or the request's last
+      if (!from_state) before.v[e] = ho;
+      o.v[e] = fmaf(before.v[e] - h.v[e], mi.v[e], h.v[e]);
+      keep.v[e] = ho;
+    }
+    if (from_state) store_pack<V>(st + i, keep);
+    store_pack<V>(orow + i, o);
+  }
+}
+
 }  // namespace
 }  // namespace bc4g
 
@@ -163,4 +240,24 @@ extern "C" int bc4g_gelu(const void* in, void* out, int dtype, long total, void*
   else if (dtype == kBF16) gelu_kernel<bf16_t><<<grid_for(total), kBlock, 0, s>>>(static_cast<const bf16_t*>(in), static_cast<bf16_t*>(out), total);
   else return fail("gelu: unknown dtype %d", dtype);
   return check_launch("gelu");
+}
+
+extern "C" int bc4g_rmsnorm_shift(const float* x, const float* w, const float* mix, void* out, void* state, int dtype,
+                                  const int32_t* row_seq, const int32_t* seq_start, const int32_t* seq_slots, int n_rows,
+                                  int hidden, float eps, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && hidden > 0 && x && w && mix && out && state && row_seq && seq_start && seq_slots,
+               "rmsnorm_shift: bad arguments rows=%d H=%d", n_rows, hidden);
+  if (n_rows == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const bool four = hidden % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(mix) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(state) % 16 == 0;
+#define BC4G_SHIFT(T, V)                                                                                                    \
+  rmsnorm_shift_kernel<T, V><<<n_rows, kBlock, 0, s>>>(x, w, mix, static_cast<T*>(out), static_cast<T*>(state), row_seq, seq_start, \
+                                                      seq_slots, hidden, eps)
+  if (dtype == kF32) { if (four) BC4G_SHIFT(float, 4); else BC4G_SHIFT(float, 1); }
+  else if (dtype == kBF16) { if (four) BC4G_SHIFT(bf16_t, 4); else BC4G_SHIFT(bf16_t, 1); }
+  else return fail("rmsnorm_shift: unknown dtype %d", dtype);
+#undef BC4G_SHIFT
+  return check_launch("rmsnorm_shift");
 }

@@ -44,6 +44,7 @@ _SIGNATURES = {
     "bc4g_gemm_skinny_prenormed": [_P, _P, _I, _I, _F, _P, _P, _I, _I, _I, _I, _P],
     "bc4g_rmsnorm_add": [_P, _P, _I, _P, _I, _I, _F, _P],
     "bc4g_xielu": [_P, _P, _I, _P, c_long, _P],
+    "bc4g_rmsnorm_shift": [_P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _F, _P],
     "bc4g_causal_conv": [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_long, _P],
     "bc4g_rglru_scan": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, c_long, _P],
     "bc4g_latent_angles": [_P, _P, _I, _I, _F, _P],

@@ -1244,6 +1244,30 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Ten
     return out
 
 
+def rmsnorm_shift(x: torch.Tensor, weight: torch.Tensor, eps: float, mix: torch.Tensor, state: torch.Tensor, ctx,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """An RMS norm of the float32 stream x [T, H] and the token shift behind it in one launch: h = norm(x) (rounded to
+    ``out_dtype``), out[t] = h[t] + (h[t - 1] - h[t]) * mix along a request's rows.  ``state`` [slots, 1, H] (``out_dtype``)
+    holds every request's last h so far -- h[-1] for its first row of this step -- and receives the last h of this step.
+    weight, mix: float32 [H]."""
+    _dev("rmsnorm_shift", x, weight, mix, state)
+    if x.dtype != torch.float32 or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError(f"rmsnorm_shift: x must be float32 [T, H], got {x.dtype} {tuple(x.shape)}")
+    t, hidden = x.shape
+    _f32("rmsnorm_shift", "weight", weight, (hidden,))
+    _f32("rmsnorm_shift", "mix", mix, (hidden,))
+    if state.dtype != out_dtype or state.dim() != 3 or tuple(state.shape[1:]) != (1, hidden) or not state.is_contiguous():
+        raise KernelError(f"rmsnorm_shift: state must be {out_dtype} [slots, 1, {hidden}], got {state.dtype} {tuple(state.shape)}")
+    if max(ctx.seq_slots, default=0) >= state.shape[0]:
+        raise KernelError(f"rmsnorm_shift: a slot beyond the state's {state.shape[0]}")
+    _check_grouping("rmsnorm_shift", ctx, t)
+    out = torch.empty((t, hidden), dtype=out_dtype, device=x.device)
+    library.call("bc4g_rmsnorm_shift", _ptr(x), _ptr(weight), _ptr(mix), _ptr(out), _ptr(state), _code(out, "rmsnorm_shift"),
+                 _ptr(ctx.row_seq), _ptr(ctx.seq_start_dev), _ptr(ctx.seq_slots_dev), t, hidden, float(eps), _stream(),
+                 cost=lambda: (8.0 * t * hidden, t * hidden * (4 + out.element_size())))
+    return out
+
+
 RGLRU_CHUNK = 64            # rows of a request that one thread of the recurrence walks
 
 

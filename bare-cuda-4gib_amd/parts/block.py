@@ -38,8 +38,13 @@ class PreNormBlock(Part):
         with handoff.reader(*after_mixer):
             if self.mixer_shift is not None:
                 pre = handoff.take(self.mixer_norm)
-                h = pre.tensor if isinstance(pre, ops.Finished) else self.mixer_norm.forward(x, ctx)
-                self.mixer.forward(self.mixer_shift.forward(h, ctx, cache.shift), ctx, cache.mixer, x, writes)
+                if isinstance(pre, ops.Finished):
+                    h = self.mixer_shift.forward(pre.tensor, ctx, cache.shift)
+                elif hasattr(self.mixer_shift, "after"):       # (norm and shift in one kernel where the two know how)
+                    h = self.mixer_shift.after(self.mixer_norm, x, ctx, cache.shift)
+                else:
+                    h = self.mixer_shift.forward(self.mixer_norm.forward(x, ctx), ctx, cache.shift)
+                self.mixer.forward(h, ctx, cache.mixer, x, writes)
             else:
                 self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
         if self.ffn is None:

@@ -47,7 +47,8 @@ class CausalConv(Part):
 class TokenShift(Part):
     """out[t] = h[t] + (h[t - 1] - h[t]) * m, element by element, along a request's rows; h[-1] = 0.  The h on the right
     are the rows as they came in.  A request's last row is its state (``tail``, in the activations' dtype), so a prompt
-    may be cut anywhere.  It is the causal convolution with the taps (m, -m) plus its input."""
+    may be cut anywhere.  It is the causal convolution with the taps (m, -m) plus its input.  ``after(norm, x, ...)`` is
+    the shift of norm(x): behind an RMS norm both are one kernel (the same state, the same roundings)."""
     category = "conv"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
@@ -55,7 +56,7 @@ class TokenShift(Part):
         if channels <= 0:
             raise ConfigError(f"token shift: {channels} channels")
         self.channels = int(channels)
-        self.w = None
+        self.w = self.m = self._norm = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {"weight": WeightSpec((self.channels,), kind="vector")}
@@ -63,12 +64,24 @@ class TokenShift(Part):
     def bind(self, tensors, rt) -> None:
         m = tensors["weight"].to(torch.float32)
         self.w = torch.stack([m, -m], dim=0).contiguous()      # by taps: the row before, the row itself
+        self.m = m.contiguous()
+        self.out_dtype = rt.act_dtype
 
     def cache_spec(self):
         return States((("tail", (1, self.channels), None),))
 
     def forward(self, h: torch.Tensor, ctx, view) -> torch.Tensor:
         return ops.causal_conv(h, self.w, view.tail, ctx, add_input=True)
+
+    def after(self, norm, x: torch.Tensor, ctx, view) -> torch.Tensor:
+        """The shift of norm(x) for the float32 stream x [T, H]."""
+        fusable = getattr(norm, "fusable", None)
+        if fusable is None or x.dim() != 2 or x.dtype != torch.float32:
+            return self.forward(norm.forward(x, ctx), ctx, view)
+        if self._norm is None or self._norm[0] is not norm:
+            g, eps = fusable()
+            self._norm = (norm, g.to(torch.float32).contiguous(), float(eps))
+        return ops.rmsnorm_shift(x, self._norm[1], self._norm[2], self.m, view.tail, ctx, self.out_dtype)
 
 
 register_part("conv", "causal", CausalConv)

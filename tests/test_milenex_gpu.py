@@ -332,6 +332,44 @@ def test_shift_and_convolution_over_portions_and_slots_used_again(dtype, taps):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C", [44, 320, 2500])
+def test_norm_and_shift_in_one_pass_over_portions_and_slots_used_again(dtype, C):
+    """The norm with a weight around zero and the token shift behind it as one kernel: requests cut into unequal portions
+    that share steps, states in slots given in another order, a slot used again by a new request; against the plain
+    functions on whole sequences, and against the two kernels one after the other."""
+    from bare_cuda_4gib_amd.csrc import ops
+    torch.manual_seed(C)
+    eps = 1e-3
+    seqs = [torch.randn(n, C) * 2.0 for n in (23, 9, 1, 14)]
+    g, m = (torch.randn(C) * 0.3), torch.rand(C)
+    want = [plain.token_shift(plain.zero_centred_norm(s.double(), g.double(), eps).to(dtype).double(), m.double()) for s in seqs]
+    state = torch.full((3, 1, C), float("nan"), dtype=dtype, device=DEV)
+    apart = torch.full((3, 1, C), float("nan"), dtype=dtype, device=DEV)
+    w, mix = (1.0 + g).to(DEV), m.to(DEV)
+    taps = torch.stack([m, -m], dim=0).contiguous().to(DEV)
+    plan = [[(0, 2, 1), (1, 0, 4)], [(0, 2, 2), (1, 0, 5), (2, 1, 1)], [(0, 2, 7)], [(0, 2, 1), (3, 0, 1)], [(0, 2, 12), (3, 0, 13)]]
+    done, got = [0, 0, 0, 0], [[] for _ in seqs]
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for step in plan:
+        ctx = step_context([n for _, _, n in step], [done[r] for r, _, _ in step], [slot for _, slot, _ in step])
+        x = torch.cat([seqs[r][done[r]:done[r] + n] for r, _, n in step]).to(DEV)
+        for r, slot, _ in step:
+            if done[r] == 0:
+                state[slot].zero_()
+                apart[slot].zero_()
+        y = ops.rmsnorm_shift(x, w, eps, mix, state, ctx, dtype)
+        two = ops.causal_conv(ops.rmsnorm(x, w, eps, dtype), taps, apart, ctx, add_input=True)
+        assert torch.allclose(y.float(), two.float(), atol=tol, rtol=tol)
+        at = 0
+        for r, _, n in step:
+            got[r].append(y[at:at + n].float().cpu().double())
+            at, done[r] = at + n, done[r] + n
+    assert torch.allclose(state.float().nan_to_num(7.0), apart.float().nan_to_num(7.0), atol=tol, rtol=tol)       # the same states
+    for r in range(len(seqs)):
+        assert torch.allclose(torch.cat(got[r]), want[r], atol=tol, rtol=tol), r
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,dim,dims,base", [(3, 8, 8, 10000.0), (2, 48, 24, 500.0), (5, 7, 6, 30.0), (1, 130, 2, 7.0), (4, 10, 0, 1.0)])
 def test_neighbours_are_rotated_then_the_head_is_divided_by_its_root_mean_square(dtype, heads, dim, dims, base):
     from bare_cuda_4gib_amd.csrc import ops
