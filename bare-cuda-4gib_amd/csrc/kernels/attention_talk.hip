@@ -71,8 +71,10 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
   __shared__ float s_s[kMaxWaves][kWave];     // a head's scores on their way from (key, piece) lanes to lane = key
   __shared__ float m_s[kMaxWaves][kWave];     // a head's mixed weights, lane = key -> every lane
   const int dimp = 32 * E4;                   // a head's queries in LDS, zeros beyond dim
+  const int hp = (n_heads + 7) / 8 * 8;       // heads in whole eights: the mixing takes eight at a time
   float* q_s = dyn;                           // [heads][dimp]
-  float* p_s = dyn + n_heads * dimp;          // [heads][64]: the tile's weights
+  float* p_s = dyn + n_heads * dimp;          // [hp][64]: the tile's weights (zeros beyond the heads)
+  float* t_s = p_s + hp * kWave;              // [heads][hp]: the mixing matrix (zeros beyond the heads)
   const int row = blockIdx.x, lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int n_waves = blockDim.x / kWave;
   const int per_kv = n_heads / n_kv_heads;
@@ -82,6 +84,9 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
     const int h = i / dimp, c = i % dimp;
     q_s[i] = c < dim ? q[row * q_row + static_cast<long>(h) * dim + c] : 0.f;
   }
+  for (int i = n_heads * kWave + threadIdx.x; i < hp * kWave; i += blockDim.x) p_s[i] = 0.f;
+  if (talk)
+    for (int i = threadIdx.x; i < n_heads * hp; i += blockDim.x) t_s[i] = i % hp < n_heads ? talk[(i / hp) * n_heads + i % hp] : 0.f;
   __syncthreads();
 
   const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -252,7 +257,11 @@ __global__ __launch_bounds__(kMaxWaves * kWave) void attention_talk_kernel(
       float mixed;
       if (talk) {
         mixed = 0.f;
-        for (int g = 0; g < n_heads; ++g) mixed = fmaf(talk[h * n_heads + g], p_s[g * kWave + lane], mixed);
+        const float* t_row = t_s + h * hp;
+        for (int g0 = 0; g0 < hp; g0 += 8) {             // (eight reads of each kind in flight together)
+#pragma unroll
+          for (int u = 0; u < 8; ++u) mixed = fmaf(t_row[g0 + u], p_s[(g0 + u) * kWave + lane], mixed);
+        }
       } else {
         mixed = p_s[h * kWave + lane];
       }
@@ -370,7 +379,8 @@ extern "C" int bc4g_attention_talk(const float* q, long q_row, const void* k_cac
   const int waves = n_heads < kMaxWaves ? n_heads : kMaxWaves;
   const int slots = (n_heads + waves - 1) / waves;
   const int by_slot = n_parts > 1 && kept && slots > 1;
-  const size_t lds = static_cast<size_t>(n_heads) * (32 * e4 + kWave) * sizeof(float);
+  const int hp = (n_heads + 7) / 8 * 8;
+  const size_t lds = (static_cast<size_t>(n_heads) * (32 * e4 + hp) + static_cast<size_t>(hp) * kWave) * sizeof(float);
   const bool v_four = vdim % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
 #define BC4G_TALK_PHASE(T, SL, E, V, PHASE)                                                                                 \
   attention_talk_kernel<T, SL, E, V><<<dim3(n_rows, n_parts, by_slot ? slots : 1), waves * kWave, lds, s>>>(                \
