@@ -92,24 +92,31 @@ class PagedHeads:
     """Keys and values per token, in pages, with head counts and sizes of their own: keys
     ``[page, key_heads, token, key_dim]``, values ``[page, value_heads, token, value_dim]`` (a token's elements side by
     side in both).  ``window`` 0 keeps every token; otherwise a query reads the last ``window`` tokens and, whatever its
-    position, the first ``keep_first`` tokens of the sequence: pages between those and the window are given back."""
+    position, the first ``keep_first`` tokens of the sequence: pages between those and the window are given back.
+    ``block`` (instead of a window): a query reads the keys of its own block of that many positions, counted from the
+    sequence's first token; pages wholly before the current block are given back."""
     key_heads: int
     key_dim: int
     value_heads: int
     value_dim: int
     window: int = 0
     keep_first: int = 0
+    block: int = 0
     per_token = True
 
     def page_tensors(self, page_tokens: int) -> Dict[str, Tuple[int, ...]]:
         return {"k": (self.key_heads, page_tokens, self.key_dim), "v": (self.value_heads, page_tokens, self.value_dim)}
 
     def group_key(self):
+        if self.block > 0:
+            return ("block", self.block)
         if self.window <= 0 or self.keep_first <= 0:
             return ("window", max(self.window, 0))
         return ("window", self.window, "first", self.keep_first)
 
     def first_kept(self, length: int) -> int:
+        if self.block > 0:
+            return length - length % self.block
         return max(0, length - self.window + 1) if self.window > 0 else 0
 
     def always_kept(self) -> int:

@@ -7,3 +7,4 @@ from .llama import LlamaConfig  # noqa: F401
 from .mamenex import MamenexConfig  # noqa: F401
 from .nagezen import NagezenConfig  # noqa: F401
 from .milenex import MilenexConfig  # noqa: F401
+from .lagusun import LagusunConfig  # noqa: F401

@@ -18,10 +18,25 @@ const char* bc4g_sources_digest();   // digest of the sources and flags the libr
 int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
                       int n_tokens, int hidden, int vocab, void* stream);
 
+// x[t, :] (+)= float(table[ids[t], :]) * factor  (add 0: stored, 1: added to what x holds)
+int bc4g_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden, int vocab,
+                    float factor, int add, void* stream);
+
 // out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w      (rmsnorm.cu:16-41)
 // x is the float residual stream; out has out_dtype; w has w_dtype.
 int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
                  int out_dtype, int n_rows, int hidden, float eps, void* stream);
+// The same with every row cut into `groups` equal consecutive parts, each divided by its own root mean square (w spans the row).
+int bc4g_rmsnorm_groups(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out, int out_dtype, int n_rows,
+                        int hidden, int groups, float eps, void* stream);
+// x = (keep ? x : 0) + scale * y + bias on the float32 stream x [n_rows, hidden] (y float32 of that shape; scale, bias float32
+// [hidden], each may be null: 1, 0), written back; with w (and out, in out_dtype) also out = the norm of the new x in
+// `groups` parts as bc4g_rmsnorm_groups computes it (stream_update.hip).
+int bc4g_stream_update(float* x, const float* y, const float* scale, const float* bias, int keep, const void* w, int w_dtype,
+                       void* out, int out_dtype, int n_rows, int hidden, int groups, float eps, void* stream);
+// out[t] = [x[t, :] | table[ids[t], :] * factor] in out_dtype, [n_tokens, 2 hidden]: the stream beside the embedding.
+int bc4g_embed_beside(const float* x, const void* table, int table_dtype, const int32_t* ids, float factor, void* out,
+                      int out_dtype, int n_tokens, int hidden, int vocab, void* stream);
 // The same for a stream whose last addition is still in parts [n_parts, n_rows, hidden] (float32, as
 // bc4g_gemm_mfma_parts leaves them): x += parts[0] + parts[1] + ... in that order, written back, then out = its norm
 // (bfloat16).  hidden a multiple of 8, at most 8192.
@@ -319,7 +334,9 @@ struct bc4g_prepare_section {
   float eps, factor;
   // pairing 0: element i turns with element i + half, 1: element 2i with element 2i + 1.  unit_after 1: after the
   // rotation the head is divided by sqrt(mean(head^2) + eps), without a weight.
-  int pairing, unit_after;
+  // norm_rows 1: the norm before the rotation is taken over the whole row -- all heads at once, mean over heads * dim --
+  // and norm_w is [heads * dim]; 0: over each head, norm_w [dim].
+  int pairing, unit_after, norm_rows;
 };
 int bc4g_heads_prepare_many(const bc4g_prepare_section* sections, int n_sections, int n_rows, void* stream);
 int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, const float* bias, const float* norm_w, float eps,
@@ -347,12 +364,15 @@ int bc4g_decay_scan(const void* q, int q_dtype, long q_row, float q_scale, const
 // divided by sqrt(mean(o^2) + eps), times factor, times act(gate) (1: silu, 2: sigmoid; gate null: none).  waves (1 to 8):
 // how many waves cut one row's keys among them.  sink [heads] (or null): exp(sink) joins every map's denominator.
 // far1, far2 [heads] (both or neither): far1 ln(1 + far2 (p - j)) is taken off the scaled score.
+// block > 0 (then window and keep_first 0): a row sees the keys of its own block of `block` positions counted from 0,
+// j <= p with j / block == p / block.  cap > 0: the scaled score becomes cap tanh(score / cap).  point [heads] (or null; then
+// no sink): no softmax -- the weight of a visible key is sigmoid(score + point[head]), nothing is normalised over keys.
 int bc4g_attention_maps(const float* q, long q_row, const void* k_cache, const void* v_cache, int cache_dtype,
                         const int32_t* block_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                         float lambda, int normalize, float eps, float factor, const void* gate, int gate_dtype, long gate_row,
                         int gate_act, void* out, int out_dtype, int n_rows, int n_heads, int n_kv_heads, int maps, int dim,
                         int vdim, int page_tokens, int window, int keep_first, float scale, int waves, const float* sink,
-                        const float* far1, const float* far2, void* stream);
+                        const float* far1, const float* far2, int block, float cap, const float* point, void* stream);
 
 // Windowed softmax attention whose heads' weights are mixed before they meet the values (attention_talk.hip): q float32
 // [T, heads, dim]; keys [page, kv_head, token, dim], values [page, kv_head, token, vdim]; a row at p sees j <= p with
@@ -381,9 +401,16 @@ int bc4g_gelu(const void* in, void* out, int dtype, long total, void* stream);
 // softmax over the experts; choice = s + correction (null: s); the experts lie in `groups` equal groups of neighbours, a
 // group counts by its largest choice, and only experts of the `keep` best groups can be chosen; the `top` largest
 // choices win (the lower index among equals).  weights float32 [T, experts]: s of the chosen, 0 elsewhere.
-// chosen int32 [T, top] (may be null).  experts at most 1024.
+// chosen int32 [T, top] (may be null).  experts at most 1024.  squash 1: s = sigmoid(logit), every expert by itself,
+// instead of the softmax.  normalize 1: the chosen experts' weights are their s divided by the sum of the chosen s
+// (+ 1e-20).  The weights are multiplied by `factor` last.
 int bc4g_moe_route(const float* logits, long logits_row, const float* correction, float* weights, int32_t* chosen,
-                   int n_rows, int experts, int groups, int keep, int top, void* stream);
+                   int n_rows, int experts, int groups, int keep, int top, int squash, int normalize, float factor,
+                   void* stream);
+// Plain units of all experts side by side, weighted: z [T, experts * ff + shared_ff] holds every expert's ff units and
+// last the shared unit's; out (may be z) = weights[t, e] * gelu(z) with the exact gelu, the shared unit's as they are.
+int bc4g_routed_gelu(const void* z, void* out, int dtype, const float* weights, int n_rows, int experts, int ff, int shared_ff,
+                     void* stream);
 // Clamped gated units of all experts side by side, weighted: gu [T, experts * 2 ff + 2 shared_ff] holds per expert its
 // ff gates, then its ff ups, and last the shared unit's gates and ups; out [T, experts * ff + shared_ff] =
 // weights[t, e] * g sigmoid(slope g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), the shared unit

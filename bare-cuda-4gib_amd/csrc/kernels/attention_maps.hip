@@ -4,6 +4,9 @@
 // scaled and gated.  Two further options, each a vector with one number a query head: a sink -- exp(sink) joins the
 // softmax's denominator, with no key and no value, never scaled -- and a penalty on distance, r1 ln(1 + r2 (p - j)),
 // taken off the scaled score.  Plain float arithmetic on float or bfloat16 caches: scores, weights and sums are float32.
+// Three more, for the whole call: a mask by blocks instead of the window (a row sees the keys of its own block of
+// `block` positions counted from 0, up to itself), a cap on the scaled score, cap tanh(score / cap), and weights that are no
+// softmax: sigmoid(score + point[head]) for every visible key by itself, no maximum, no denominator, no sink.
 //
 // A row at position p sees key j if j <= p and (window == 0 or p - j < window or j < keep_first); kept keys keep their
 // own positions (they were rotated when they were written).  One workgroup per (row, query head): the visible keys --
@@ -63,7 +66,8 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
     const int32_t* __restrict__ positions, float lambda, int normalize, float eps, float factor,
     const void* __restrict__ gate, int gate_dtype, long gate_row, int gate_act, void* __restrict__ out, int out_dtype,
     int n_heads, int n_kv_heads, int dim, int vdim, int page_tokens, int window, int keep_first, float scale,
-    const float* __restrict__ sink, const float* __restrict__ far1, const float* __restrict__ far2) {
+    const float* __restrict__ sink, const float* __restrict__ far1, const float* __restrict__ far2, int block, float cap,
+    const float* __restrict__ point) {
   __shared__ __align__(16) float q_s[MAPS][kMaxDim];
   __shared__ float p_s[kNW][MAPS][kWave];
   __shared__ long v_at[kNW][kWave];           // where every key of the wave's tile has its values
@@ -81,7 +85,8 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
       q_s[m][c] = c < dim ? q[row * q_row + (static_cast<long>(head) * MAPS + m) * dim + c] : 0.f;
   __syncthreads();
 
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = block > 0 ? pos - pos % block : (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const float lift = point ? point[head] : 0.f;
   const int kept = window > 0 ? (keep_first < first ? keep_first : first) : 0;      // kept keys before the window
   const int total = kept + (pos - first + 1);
   const float pen1 = far1 ? far1[head] : 0.f, pen2 = far1 ? far2[head] : 0.f;
@@ -160,6 +165,12 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
       }
       float sc = dot * scale;
       if (far1) sc -= pen1 * log1pf(pen2 * static_cast<float>(pos - j));
+      if (cap > 0.f) sc = cap * tanhf(sc / cap);
+      if (point) {                                           // a weight a key by itself: nothing to keep up with
+        p_s[wave][m][lane] = seen ? 1.0f / (1.0f + expf(-(sc + lift))) : 0.f;
+        mx[m] = 0.f;
+        continue;
+      }
       if (!seen) sc = -INFINITY;
       const float m_new = fmaxf(mx[m], wave_max(sc));       // finite: the tile's first key is visible
       const float p = seen ? expf(sc - m_new) : 0.f;
@@ -234,7 +245,11 @@ __global__ __launch_bounds__(kNW * kWave) void attention_maps_kernel(
       mx[m] = top;                                       // (what the merged sums are counted from)
     }
   }
-  if (sink) {                                            // the sink: a term of the denominator, with no value
+  if (point) {                                           // (the parts' weights are finished: they were added up as they are)
+#pragma unroll
+    for (int m = 0; m < MAPS; ++m) sum[m] = 1.0f;
+  }
+  if (sink && !point) {                                  // the sink: a term of the denominator, with no value
     const float sk = sink[head];
 #pragma unroll
     for (int m = 0; m < MAPS; ++m) {
@@ -277,7 +292,8 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
                                    const void* gate, int gate_dtype, long gate_row, int gate_act, void* out, int out_dtype,
                                    int n_rows, int n_heads, int n_kv_heads, int maps, int dim, int vdim, int page_tokens,
                                    int window, int keep_first, float scale, int waves, const float* sink,
-                                   const float* far1, const float* far2, void* stream) {
+                                   const float* far1, const float* far2, int block, float cap, const float* point,
+                                   void* stream) {
   BC4G_REQUIRE(waves >= 1 && waves <= kMaxWaves, "attention_maps: %d waves a row (1 to %d)", waves, kMaxWaves);
   BC4G_REQUIRE(n_rows >= 0 && n_heads > 0 && n_heads <= 65535 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                "attention_maps: bad sizes T=%d heads=%d/%d", n_rows, n_heads, n_kv_heads);
@@ -292,6 +308,9 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
                (!gate || gate_dtype == kF32 || gate_dtype == kBF16),
                "attention_maps: a tensor is missing, a row is shorter than its heads, or a dtype is unknown");
   BC4G_REQUIRE((far1 == nullptr) == (far2 == nullptr), "attention_maps: the distance penalty needs both of its vectors");
+  BC4G_REQUIRE(block >= 0 && (block == 0 || (window == 0 && keep_first == 0)) && cap >= 0.f && !(point && sink),
+               "attention_maps: block=%d beside window=%d, keep_first=%d; cap=%g; weights without a softmax have no sink", block,
+               window, keep_first, static_cast<double>(cap));
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(n_rows, n_heads);
@@ -306,7 +325,7 @@ extern "C" int bc4g_attention_maps(const float* q, long q_row, const void* k_cac
   attention_maps_kernel<T, M, W, V, E><<<grid, waves * kWave, 0, s>>>(q, q_row, static_cast<const T*>(k_cache), static_cast<const T*>(v_cache), \
                                                      block_table, table_stride, row_seq, positions, lambda, normalize, eps, \
                                                      factor, gate, gate_dtype, gate_row, gate_act, out, out_dtype, n_heads,  \
-                                                     n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale, sink, far1, far2)
+                                                     n_kv_heads, dim, vdim, page_tokens, window, keep_first, scale, sink, far1, far2, block, cap, point)
   if (cache_dtype == kF32) {
     if (maps == 1) BC4G_MAPS(float, 1); else BC4G_MAPS(float, 2);
   } else if (cache_dtype == kBF16) {

@@ -73,7 +73,19 @@ __global__ __launch_bounds__(kWave) void heads_prepare_kernel(const PrepareSecti
     ss = fmaf(v, v, ss);
   }
   float scale = 1.0f;
-  if (norm_w) scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dim) + p.eps);
+  if (norm_w && p.norm_rows) {      // the mean square of the whole row, all heads at once; the weight spans the row too
+    const int width = p.heads * dim;
+    float all = 0.f;
+    for (int c = lane; c < width; c += kWave) {
+      float v = load_any(p.in, p.in_dtype, row * p.in_row + c);
+      if (bias) v += bias[c];
+      all = fmaf(v, v, all);
+    }
+    scale = 1.0f / sqrtf(wave_sum(all) / static_cast<float>(width) + p.eps);
+    norm_w += static_cast<long>(head) * dim;
+  } else if (norm_w) {
+    scale = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dim) + p.eps);
+  }
   __syncthreads();
   long base;
   if (p.slot_map) {
@@ -369,7 +381,7 @@ extern "C" int bc4g_heads_prepare(const void* in, int in_dtype, long in_row, con
                                   const int32_t* slot_map, int page_tokens, long page_stride, long head_stride,
                                   long token_stride, int n_rows, int heads, int dim, void* stream) {
   const bc4g_prepare_section one{in, bias, norm_w, table, out, slot_map, in_row, out_row, page_stride, head_stride, token_stride,
-                                 in_dtype, out_dtype, half, page_tokens, heads, dim, eps, factor};
+                                 in_dtype, out_dtype, half, page_tokens, heads, dim, eps, factor, 0, 0, 0};
   return bc4g_heads_prepare_many(&one, 1, n_rows, stream);
 }
 

@@ -17,14 +17,14 @@ constexpr int kBlock = 256;
 // ---- embedding -------------------------------------------------------------
 template <typename TT>
 __global__ void embed_gather_kernel(const TT* __restrict__ table, const int32_t* __restrict__ ids,
-                                    float* __restrict__ out, int hidden, int add) {
+                                    float* __restrict__ out, int hidden, int add, float factor) {
   const size_t row = blockIdx.x;
   const TT* src = table + static_cast<size_t>(ids[row]) * hidden;
   float* dst = out + row * hidden;
   if (add) {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] += to_float(src[i]) * factor;
   } else {
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * factor;
   }
 }
 
@@ -32,10 +32,13 @@ __global__ void embed_gather_kernel(const TT* __restrict__ table, const int32_t*
 // eps is added to the mean square; sum and rsqrt in float.
 template <typename TW, typename TO>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
-                               const TW* __restrict__ w, TO* __restrict__ out, int hidden, float eps) {
+                               const TW* __restrict__ w, TO* __restrict__ out, int hidden, float eps, int groups) {
+  // (a workgroup is one of a row's `groups` equal consecutive parts, `hidden` elements each, normed by itself)
   __shared__ float scratch[16];
-  const size_t src_row = rows ? static_cast<size_t>(rows[blockIdx.x]) : blockIdx.x;
-  const float* xr = x + src_row * hidden;
+  const size_t row = blockIdx.x / groups, part = blockIdx.x % groups;
+  const size_t src_row = rows ? static_cast<size_t>(rows[row]) : row;
+  const float* xr = x + (src_row * groups + part) * hidden;
+  w += part * hidden;
   TO* orow = out + static_cast<size_t>(blockIdx.x) * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
@@ -55,10 +58,12 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __res
 template <typename TW, typename TO, int CHUNKS>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
                                                            const TW* __restrict__ w, TO* __restrict__ out, int hidden,
-                                                           float eps) {
+                                                           float eps, int groups) {
   __shared__ float scratch[16];
-  const size_t src_row = rows ? static_cast<size_t>(rows[blockIdx.x]) : blockIdx.x;
-  const float* xr = x + src_row * hidden;
+  const size_t row = blockIdx.x / groups, part = blockIdx.x % groups;
+  const size_t src_row = rows ? static_cast<size_t>(rows[row]) : row;
+  const float* xr = x + (src_row * groups + part) * hidden;
+  w += part * hidden;
   TO* orow = out + static_cast<size_t>(blockIdx.x) * hidden;
   float v[CHUNKS][8];
   float ss = 0.f;
@@ -618,15 +623,15 @@ int grid_for(long total) {
 using namespace bc4g;
 
 static int embed_rows(const char* what, const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens,
-                      int hidden, int vocab, int add, void* stream) {
+                      int hidden, int vocab, int add, float factor, void* stream) {
   BC4G_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0 && table && ids && out, "%s: bad arguments T=%d H=%d V=%d", what,
                n_tokens, hidden, vocab);
   if (n_tokens == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (table_dtype == kF32) {
-    embed_gather_kernel<float><<<n_tokens, kBlock, 0, s>>>(static_cast<const float*>(table), ids, out, hidden, add);
+    embed_gather_kernel<float><<<n_tokens, kBlock, 0, s>>>(static_cast<const float*>(table), ids, out, hidden, add, factor);
   } else if (table_dtype == kBF16) {
-    embed_gather_kernel<bf16_t><<<n_tokens, kBlock, 0, s>>>(static_cast<const bf16_t*>(table), ids, out, hidden, add);
+    embed_gather_kernel<bf16_t><<<n_tokens, kBlock, 0, s>>>(static_cast<const bf16_t*>(table), ids, out, hidden, add, factor);
   } else {
     return fail("%s: unknown table dtype %d", what, table_dtype);
   }
@@ -635,30 +640,44 @@ static int embed_rows(const char* what, const void* table, int table_dtype, cons
 
 extern "C" int bc4g_embed_gather(const void* table, int table_dtype, const int32_t* ids, float* out,
                                  int n_tokens, int hidden, int vocab, void* stream) {
-  return embed_rows("embed_gather", table, table_dtype, ids, out, n_tokens, hidden, vocab, 0, stream);
+  return embed_rows("embed_gather", table, table_dtype, ids, out, n_tokens, hidden, vocab, 0, 1.0f, stream);
+}
+
+extern "C" int bc4g_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
+                               int vocab, float factor, int add, void* stream) {
+  return embed_rows(add ? "embed_add" : "embed_gather", table, table_dtype, ids, out, n_tokens, hidden, vocab, add ? 1 : 0, factor,
+                    stream);
 }
 
 extern "C" int bc4g_embed_add(const void* table, int table_dtype, const int32_t* ids, float* out, int n_tokens, int hidden,
                               int vocab, void* stream) {
-  return embed_rows("embed_add", table, table_dtype, ids, out, n_tokens, hidden, vocab, 1, stream);
+  return embed_rows("embed_add", table, table_dtype, ids, out, n_tokens, hidden, vocab, 1, 1.0f, stream);
 }
 
 extern "C" int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
                             int out_dtype, int n_rows, int hidden, float eps, void* stream) {
-  BC4G_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", n_rows, hidden);
+  return bc4g_rmsnorm_groups(x, rows, w, w_dtype, out, out_dtype, n_rows, hidden, 1, eps, stream);
+}
+
+extern "C" int bc4g_rmsnorm_groups(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out, int out_dtype,
+                                   int n_rows, int width, int groups, float eps, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && width > 0 && groups > 0 && width % groups == 0 && static_cast<long>(n_rows) * groups < (1L << 31),
+               "rmsnorm: bad sizes rows=%d H=%d in %d groups", n_rows, width, groups);
   if (n_rows == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int hidden = width / groups;      // a workgroup norms one part
+  n_rows *= groups;
   // widths that are a multiple of 8, up to 8,192: the row stays in registers
   const int chunks = hidden % 8 == 0 ? (hidden + 2047) / 2048 : 0;
 #define BC4G_RMS(TW, TO)                                                                                    \
   do {                                                                                                      \
     const TW* wp = static_cast<const TW*>(w);                                                               \
     TO* op = static_cast<TO*>(out);                                                                         \
-    if (chunks == 1) rmsnorm_rows_kernel<TW, TO, 1><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps);      \
-    else if (chunks == 2) rmsnorm_rows_kernel<TW, TO, 2><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps); \
+    if (chunks == 1) rmsnorm_rows_kernel<TW, TO, 1><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps, groups);      \
+    else if (chunks == 2) rmsnorm_rows_kernel<TW, TO, 2><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps, groups); \
     else if (chunks == 3 || chunks == 4)                                                                    \
-      rmsnorm_rows_kernel<TW, TO, 4><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps);                   \
-    else rmsnorm_kernel<TW, TO><<<n_rows, kBlock, 0, s>>>(x, rows, wp, op, hidden, eps);                     \
+      rmsnorm_rows_kernel<TW, TO, 4><<<n_rows, 256, 0, s>>>(x, rows, wp, op, hidden, eps, groups);                   \
+    else rmsnorm_kernel<TW, TO><<<n_rows, kBlock, 0, s>>>(x, rows, wp, op, hidden, eps, groups);                     \
   } while (0)
   if (w_dtype == kF32 && out_dtype == kF32) BC4G_RMS(float, float);
   else if (w_dtype == kF32 && out_dtype == kBF16) BC4G_RMS(float, bf16_t);

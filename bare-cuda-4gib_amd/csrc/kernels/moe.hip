@@ -5,6 +5,10 @@
 //               chosen (the others count as minus infinity, not as zero: a choice may be negative); the largest `top`
 //               choices win, the lower index among equals.  Out: a row of weights over all experts -- s of the chosen, as
 //               it is, zero elsewhere -- and the chosen experts' indices.
+//               With `squash` s = sigmoid(logit), every expert by itself; with `normalize` the chosen experts' weights are
+//               their s divided by the sum of the chosen s (+ 1e-20); the weights are multiplied by a factor last.
+//   routed_gelu every expert's plain unit (the exact gelu) on its part of one wide product's row, times the row's weight for
+//               that expert; a shared unit at the end counts as it is.
 //   routed_glu  every expert's clamped gated unit on its part of one wide product's row, times the row's weight for that
 //               expert (zero for the experts the row did not choose), and a shared unit with a gate per row at the end:
 //               what one product over all experts' down matrices then adds up is the weighted sum of the chosen experts.
@@ -23,22 +27,28 @@ constexpr int kBlock = 256;
 // One wave a row.
 __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restrict__ logits, long logits_row,
                                                           const float* __restrict__ correction, float* __restrict__ weights,
-                                                          int32_t* __restrict__ chosen, int experts, int groups, int keep, int top) {
+                                                          int32_t* __restrict__ chosen, int experts, int groups, int keep, int top,
+                                                          int squash, int normalize, float factor) {
   __shared__ float s_s[kMaxExperts];        // the scores
   __shared__ float c_s[kMaxExperts];        // the choices (minus infinity once taken, or outside the kept groups)
   __shared__ float g_s[kMaxExperts];        // the groups' largest choices
   const int row = blockIdx.x, lane = threadIdx.x;
   const float* z = logits + row * logits_row;
-  float top_z = -INFINITY;
-  for (int e = lane; e < experts; e += kWave) top_z = fmaxf(top_z, z[e]);
-  top_z = wave_max(top_z);
-  float sum = 0.f;
-  for (int e = lane; e < experts; e += kWave) {
-    const float p = expf(z[e] - top_z);
-    s_s[e] = p;
-    sum += p;
+  float sum = 1.0f;
+  if (squash) {
+    for (int e = lane; e < experts; e += kWave) s_s[e] = 1.0f / (1.0f + expf(-z[e]));
+  } else {
+    float top_z = -INFINITY;
+    for (int e = lane; e < experts; e += kWave) top_z = fmaxf(top_z, z[e]);
+    top_z = wave_max(top_z);
+    sum = 0.f;
+    for (int e = lane; e < experts; e += kWave) {
+      const float p = expf(z[e] - top_z);
+      s_s[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
   }
-  sum = wave_sum(sum);
   const int per = experts / groups;
   for (int e = lane; e < experts; e += kWave) {
     const float s = s_s[e] / sum;
@@ -62,6 +72,7 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
       for (int i = 0; i < per; ++i) c_s[g * per + i] = -INFINITY;
   }
   __syncthreads();
+  float picked = 0.f;                                          // the chosen experts' scores, added up in the order of choice
   for (int n = 0; n < top; ++n) {
     float best = -INFINITY;
     int at = experts;
@@ -74,12 +85,35 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
       if (other > best || (other == best && other_at < at)) best = other, at = other_at;
     }
     if (at >= experts) break;                                 // fewer experts left than asked for
+    picked += s_s[at];
     if (lane == 0) {
-      weights[static_cast<long>(row) * experts + at] = s_s[at];
+      weights[static_cast<long>(row) * experts + at] = s_s[at] * (normalize ? 1.0f : factor);
       if (chosen) chosen[static_cast<long>(row) * top + n] = at;
       c_s[at] = -INFINITY;
     }
     __syncthreads();
+  }
+  if (normalize) {                                            // (the row's weights are this wave's own writes)
+    const float by = factor / (picked + 1e-20f);
+    for (int e = lane; e < experts; e += kWave) {
+      const float w = weights[static_cast<long>(row) * experts + e];
+      if (w != 0.f) weights[static_cast<long>(row) * experts + e] = w * by;
+    }
+  }
+}
+
+__device__ inline float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+
+template <typename T>
+__global__ void routed_gelu_kernel(const T* __restrict__ z, T* __restrict__ out, const float* __restrict__ weights, long total,
+                                   int experts, int ff, int shared_ff) {
+  const int row_width = experts * ff + shared_ff;
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
+  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total; i += stride) {
+    const long r = i / row_width;
+    const int c = static_cast<int>(i - r * row_width);
+    const float w = c < experts * ff ? weights[r * experts + c / ff] : 1.0f;
+    out[i] = from_float<T>(w != 0.f ? w * gelu_erf(to_float(z[i])) : 0.f);
   }
 }
 
@@ -122,15 +156,38 @@ __global__ void routed_glu_kernel(const T* __restrict__ gu, T* __restrict__ out,
 using namespace bc4g;
 
 extern "C" int bc4g_moe_route(const float* logits, long logits_row, const float* correction, float* weights, int32_t* chosen,
-                              int n_rows, int experts, int groups, int keep, int top, void* stream) {
+                              int n_rows, int experts, int groups, int keep, int top, int squash, int normalize, float factor,
+                              void* stream) {
   BC4G_REQUIRE(n_rows >= 0 && experts > 0 && experts <= kMaxExperts && logits && weights && logits_row >= experts,
                "moe_route: bad arguments rows=%d experts=%d (at most %d)", n_rows, experts, kMaxExperts);
   BC4G_REQUIRE(groups > 0 && experts % groups == 0 && keep > 0 && keep <= groups && top > 0 && top <= experts,
                "moe_route: %d experts in %d groups of which %d are kept, %d chosen", experts, groups, keep, top);
   if (n_rows == 0) return 0;
   moe_route_kernel<<<n_rows, kWave, 0, static_cast<hipStream_t>(stream)>>>(logits, logits_row, correction, weights, chosen,
-                                                                           experts, groups, keep, top);
+                                                                           experts, groups, keep, top, squash, normalize,
+                                                                           factor);
   return check_launch("moe_route");
+}
+
+extern "C" int bc4g_routed_gelu(const void* z, void* out, int dtype, const float* weights, int n_rows, int experts, int ff,
+                                int shared_ff, void* stream) {
+  BC4G_REQUIRE(n_rows >= 0 && experts >= 0 && ff >= 0 && shared_ff >= 0 && experts * ff + shared_ff > 0 && z && out,
+               "routed_gelu: bad arguments rows=%d experts=%d ff=%d shared=%d", n_rows, experts, ff, shared_ff);
+  BC4G_REQUIRE(experts == 0 || weights, "routed_gelu: the weights are missing");
+  const long total = static_cast<long>(n_rows) * (static_cast<long>(experts) * ff + shared_ff);
+  if (total == 0) return 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const long blocks = (total + kBlock - 1) / kBlock;
+  const int grid = static_cast<int>(blocks > 65535 ? 65535 : blocks);
+  if (dtype == kF32)
+    routed_gelu_kernel<float><<<grid, kBlock, 0, s>>>(static_cast<const float*>(z), static_cast<float*>(out), weights, total,
+                                                      experts, ff, shared_ff);
+  else if (dtype == kBF16)
+    routed_gelu_kernel<bf16_t><<<grid, kBlock, 0, s>>>(static_cast<const bf16_t*>(z), static_cast<bf16_t*>(out), weights, total,
+                                                       experts, ff, shared_ff);
+  else
+    return fail("routed_gelu: unknown dtype %d", dtype);
+  return check_launch("routed_gelu");
 }
 
 extern "C" int bc4g_routed_glu(const void* gu, void* out, int dtype, const float* weights, const float* shared_logit,

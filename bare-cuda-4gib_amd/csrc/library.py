@@ -17,7 +17,11 @@ _F = c_float
 # name -> argument types (every function returns int status, except where noted)
 _SIGNATURES = {
     "bc4g_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _P],
+    "bc4g_embed_rows": [_P, _I, _P, _P, _I, _I, _I, _F, _I, _P],
     "bc4g_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _I, _F, _P],
+    "bc4g_rmsnorm_groups": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
+    "bc4g_stream_update": [_P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _F, _P],
+    "bc4g_embed_beside": [_P, _P, _I, _P, _F, _P, _I, _I, _I, _I, _P],
     "bc4g_rmsnorm_sum": [_P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _P],
     "bc4g_gemm_mfma_parts": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
     "bc4g_gemm_mfma_swiglu_scaled": [_P, _P, _I, _I, _F, _P, _I, _P, _I, _I, _I, _P],
@@ -62,12 +66,13 @@ _SIGNATURES = {
     "bc4g_decay_scan": [_P, _I, c_long, _F, _P, _I, c_long, _P, _I, c_long, _P, _P, _I, c_long, _P, _F, _P, _P, _P, _P, _P, _P, _P,
                         _I, _I, _I, _I, _I, _I, _P],
     "bc4g_attention_maps": [_P, c_long, _P, _P, _I, _P, _I, _P, _P, _F, _I, _F, _F, _P, _I, c_long, _I, _P, _I,
-                            _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, _P],
+                            _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, _I, _F, _P, _P],
     "bc4g_attention_talk": [_P, c_long, _P, _P, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, c_long, _P, _I,
                             _I, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, c_long, _P],
     "bc4g_embed_add": [_P, _I, _P, _P, _I, _I, _I, _P],
     "bc4g_gelu": [_P, _P, _I, c_long, _P],
-    "bc4g_moe_route": [_P, c_long, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "bc4g_moe_route": [_P, c_long, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P],
+    "bc4g_routed_gelu": [_P, _P, _I, _P, _I, _I, _I, _I, _P],
     "bc4g_routed_glu": [_P, _P, _I, _P, _P, c_long, _F, _F, _F, _I, _I, _I, _I, _P],
     "bc4g_attention_latent_mfma": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 }

@@ -84,8 +84,8 @@ def _tiled_cost(m: int, n: int, k: int, out_bytes: float, qkv: bool = False):
     return cost
 
 
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t, :] = float(table[ids[t], :]); ids must already be known to lie in [0, vocab)."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, factor: float = 1.0) -> torch.Tensor:
+    """out[t, :] = float(table[ids[t], :]) * factor; ids must already be known to lie in [0, vocab)."""
     _dev("embed_gather", table, ids, out)
     vocab, hidden = table.shape
     n = ids.numel()
@@ -94,28 +94,72 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Ten
         out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
     elif out.dtype != torch.float32 or tuple(out.shape) != (n, hidden):
         raise KernelError(f"embed_gather: out must be float32 [{n}, {hidden}]")
-    library.call("bc4g_embed_gather", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out),
-                 n, hidden, vocab, _stream(), cost=lambda: (0.0, n * hidden * (table.element_size() + 4)))
+    library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out),
+                 n, hidden, vocab, float(factor), 0, _stream(), cost=lambda: (0.0, n * hidden * (table.element_size() + 4)))
     return out
 
 
-def embed_add(table: torch.Tensor, ids: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    """x[t, :] += float(table[ids[t], :]) in place on the float32 stream x [T, H]."""
+def embed_add(table: torch.Tensor, ids: torch.Tensor, x: torch.Tensor, factor: float = 1.0) -> torch.Tensor:
+    """x[t, :] += float(table[ids[t], :]) * factor in place on the float32 stream x [T, H]."""
     _dev("embed_add", table, ids, x)
     vocab, hidden = table.shape
     n = ids.numel()
     _i32("embed_add", "ids", ids, n)
     if x.dtype != torch.float32 or tuple(x.shape) != (n, hidden) or not x.is_contiguous():
         raise KernelError(f"embed_add: x must be float32 [{n}, {hidden}], got {x.dtype} {tuple(x.shape)}")
-    library.call("bc4g_embed_add", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, _stream(),
-                 cost=lambda: (1.0 * n * hidden, n * hidden * (table.element_size() + 8)))
+    library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, float(factor), 1,
+                 _stream(), cost=lambda: (1.0 * n * hidden, n * hidden * (table.element_size() + 8)))
     return x
 
 
+def embed_beside(x: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, out_dtype: torch.dtype, factor: float = 1.0) -> torch.Tensor:
+    """[T, 2 H] in ``out_dtype``: row t is the float32 stream's row x[t, :] followed by table[ids[t], :] * factor -- the
+    operand of a product over the stream and the embedding of the same token."""
+    _dev("embed_beside", x, table, ids)
+    vocab, hidden = table.shape
+    n = ids.numel()
+    _i32("embed_beside", "ids", ids, n)
+    if x.dtype != torch.float32 or tuple(x.shape) != (n, hidden):
+        raise KernelError(f"embed_beside: x must be float32 [{n}, {hidden}], got {x.dtype} {tuple(x.shape)}")
+    out = torch.empty((n, 2 * hidden), dtype=out_dtype, device=x.device)
+    library.call("bc4g_embed_beside", _ptr(x), _ptr(table), _code(table, "embed_beside"), _ptr(ids), float(factor), _ptr(out),
+                 _code(out, "embed_beside"), n, hidden, vocab, _stream(),
+                 cost=lambda: (1.0 * n * hidden, n * hidden * (4 + table.element_size() + 2 * out.element_size())))
+    return out
+
+
+def stream_update(x: torch.Tensor, y: torch.Tensor, scale: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                  keep: bool = True, norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, groups: int = 1,
+                  out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """x = (x if keep else 0) + scale * y + bias in place on the float32 stream x [T, H]; y float32 [T, H]; scale and bias
+    float32 [H] (absent: 1 and 0).  With ``norm_weight`` [H] the new x's norm in ``groups`` parts (see rmsnorm) is returned in
+    ``out_dtype`` -- what the stream's next reader would compute."""
+    _dev("stream_update", x, y, scale, bias, norm_weight)
+    if x.dtype != torch.float32 or x.dim() != 2 or y.dtype != torch.float32 or y.shape != x.shape or y.data_ptr() == x.data_ptr():
+        raise KernelError(f"stream_update: x and y must be two float32 [T, H] tensors, got {x.dtype} {tuple(x.shape)} and "
+                          f"{y.dtype} {tuple(y.shape)}")
+    t, hidden = x.shape
+    _f32("stream_update", "scale", scale, (hidden,))
+    _f32("stream_update", "bias", bias, (hidden,))
+    if groups <= 0 or hidden % groups:
+        raise KernelError(f"stream_update: {hidden} channels do not fall into {groups} equal groups")
+    out = None
+    if norm_weight is not None:
+        if tuple(norm_weight.shape) != (hidden,):
+            raise KernelError(f"stream_update: the norm's weight must be [{hidden}], got {tuple(norm_weight.shape)}")
+        out = torch.empty((t, hidden), dtype=out_dtype or torch.float32, device=x.device)
+    library.call("bc4g_stream_update", _ptr(x), _ptr(y), _ptr(scale), _ptr(bias), 1 if keep else 0, _ptr(norm_weight),
+                 _code(norm_weight, "stream_update") if norm_weight is not None else F32, _ptr(out),
+                 _code(out, "stream_update") if out is not None else F32, t, hidden, int(groups), float(eps), _stream(),
+                 cost=lambda: (6.0 * t * hidden, t * hidden * (12 + (out.element_size() if out is not None else 0))))
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
-            rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
+            rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, groups: int = 1) -> torch.Tensor:
     """RMSNorm of rows of the float residual stream x [T, H]; with ``rows`` (int32
-    indices, the first n_rows are used) only those rows are normed."""
+    indices, the first n_rows are used) only those rows are normed.  ``groups``: a row is cut into that many equal
+    consecutive parts and each is divided by its own root mean square; the weight spans the row."""
     _dev("rmsnorm", x, weight, rows)
     if x.dtype != torch.float32 or x.dim() != 2:
         raise KernelError(f"rmsnorm: x must be float32 [T, H], got {x.dtype} {tuple(x.shape)}")
@@ -127,9 +171,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     else:
         n = rows.numel() if n_rows is None else n_rows
         _i32("rmsnorm", "rows", rows, n)
+    if groups <= 0 or hidden % groups:
+        raise KernelError(f"rmsnorm: {hidden} channels do not fall into {groups} equal groups")
     out = torch.empty((n, hidden), dtype=out_dtype, device=x.device)
-    library.call("bc4g_rmsnorm", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
-                 _code(out, "rmsnorm"), n, hidden, float(eps), _stream(),
+    library.call("bc4g_rmsnorm_groups", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
+                 _code(out, "rmsnorm"), n, hidden, int(groups), float(eps), _stream(),
                  cost=lambda: (3.0 * n * hidden, n * hidden * (4 + out.element_size()) + hidden * weight.element_size()))
     return out
 
@@ -1554,24 +1600,25 @@ class _PrepareSection(ctypes.Structure):
                 ("page_stride", ctypes.c_long), ("head_stride", ctypes.c_long), ("token_stride", ctypes.c_long),
                 ("in_dtype", ctypes.c_int), ("out_dtype", ctypes.c_int), ("half", ctypes.c_int), ("page_tokens", ctypes.c_int),
                 ("heads", ctypes.c_int), ("dim", ctypes.c_int), ("eps", ctypes.c_float), ("factor", ctypes.c_float),
-                ("pairing", ctypes.c_int), ("unit_after", ctypes.c_int)]
+                ("pairing", ctypes.c_int), ("unit_after", ctypes.c_int), ("norm_rows", ctypes.c_int)]
 
 
 def heads_section(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                   norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, table: Optional[torch.Tensor] = None,
                   factor: float = 1.0, slot_map: Optional[torch.Tensor] = None, page_tokens: int = 0,
-                  neighbours: bool = False, unit_after: bool = False):
+                  neighbours: bool = False, unit_after: bool = False, norm_rows: bool = False):
     """One section for heads_prepare_many: every head of x [T, heads * dim] (may be a part of wider rows): + bias, RMS norm
     over the head with ``norm_weight`` [dim], rotation by ``table`` [T, half, 2] (element i with element i + half, or with
     ``neighbours`` element 2i with element 2i + 1), with ``unit_after`` division by sqrt(mean(head^2) + eps) of the head as
-    it stands then, times ``factor``.  ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache
+    it stands then, times ``factor``.  With ``norm_rows`` the norm before the rotation is taken over the whole row, all heads
+    at once, and ``norm_weight`` is [heads * dim].  ``out``: [T, heads, dim] (float32 or bfloat16), or with ``slot_map`` a cache
     [pages, heads, page_tokens, dim] whose slot page * page_tokens + offset receives the row.  Checked here; the tensors
     must live until the launch."""
     _dev("heads_prepare", bias, norm_weight, table, out, slot_map)
     in_row = _part_of_rows("heads_prepare", "x", x, heads * dim)
     t = x.shape[0]
     _f32("heads_prepare", "bias", bias, (heads * dim,))
-    _f32("heads_prepare", "norm_weight", norm_weight, (dim,))
+    _f32("heads_prepare", "norm_weight", norm_weight, (heads * dim,) if norm_rows else (dim,))
     half = 0
     if table is not None:
         half = table.shape[1]
@@ -1590,7 +1637,8 @@ def heads_section(x: torch.Tensor, heads: int, dim: int, out: torch.Tensor, *, b
         out_row = heads * dim
     section = _PrepareSection(_ptr(x), _ptr(bias), _ptr(norm_weight), _ptr(table), _ptr(out), _ptr(slot_map), in_row, out_row,
                               page_stride, head_stride, token_stride, _code(x, "heads_prepare"), _code(out, "heads_prepare"), half,
-                              page_tokens, heads, dim, float(eps), float(factor), 1 if neighbours else 0, 1 if unit_after else 0)
+                              page_tokens, heads, dim, float(eps), float(factor), 1 if neighbours else 0, 1 if unit_after else 0,
+                              1 if norm_rows and norm_weight is not None else 0)
     return section, t, t * heads * dim, x.element_size() + out.element_size()
 
 
@@ -1692,16 +1740,24 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    n_heads: int, n_kv_heads: int, maps: int, dim: int, vdim: int, window: int, keep_first: int, scale: float, *,
                    lam: float = 0.0, normalize: bool = False, eps: float = 0.0, factor: float = 1.0,
                    gate: Optional[torch.Tensor] = None, act: int = ACT_SIGMOID, waves: int = 0,
-                   sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                   sink: Optional[torch.Tensor] = None, far: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                   block: int = 0, cap: float = 0.0, point: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention with ``maps`` (1 or 2) score maps per query head over the same values: q float32
     [T, n_heads, maps, dim]; keys [pages, n_kv_heads * maps, page_tokens, dim], values [pages, n_kv_heads, page_tokens, vdim].
     A row at position p sees key j <= p if p - j < window or j < keep_first (window 0: every key).  o = a1 - lam a2,
     with ``normalize`` divided by sqrt(mean(o^2) + eps) over the head, times ``factor`` and act(gate); [T, n_heads * vdim].
     ``waves``: how many waves cut one row's keys among them (0: chosen here -- one where the rows fill the GPU, up to
     eight where few rows walk long contexts).  ``sink`` (float32 [n_heads]): exp(sink) joins every map's denominator, with
-    no key and no value.  ``far`` = (r1, r2), float32 [n_heads] each: r1 ln(1 + r2 (p - j)) is taken off the scaled score."""
-    _dev("attention_maps", q, k_cache, v_cache, block_table, sink, *(far or ()))
+    no key and no value.  ``far`` = (r1, r2), float32 [n_heads] each: r1 ln(1 + r2 (p - j)) is taken off the scaled score.
+    ``block`` (instead of a window): a row sees the keys j <= p of its own block of that many positions, counted from 0.
+    ``cap``: the scaled score becomes cap tanh(score / cap).  ``point`` (float32 [n_heads], no sink then): no softmax -- a
+    visible key weighs sigmoid(score + point[head]), nothing is normalised over keys."""
+    _dev("attention_maps", q, k_cache, v_cache, block_table, sink, point, *(far or ()))
     _f32("attention_maps", "sink", sink, (n_heads,))
+    _f32("attention_maps", "point", point, (n_heads,))
+    if block < 0 or (block > 0 and (window > 0 or keep_first > 0)) or cap < 0 or (point is not None and sink is not None):
+        raise KernelError(f"attention_maps: block {block} beside window {window} and {keep_first} kept keys, cap {cap}, or a sink "
+                          "beside weights that are no softmax")
     for v in far or ():
         _f32("attention_maps", "far", v, (n_heads,))
     t = q.shape[0]
@@ -1724,7 +1780,10 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         keys = pairs = 0
         for s in range(ctx.n_seqs):
             cached, new = int(ctx.seq_ctx[s]), int(ctx.seq_start[s + 1] - ctx.seq_start[s])
-            if window > 0:
+            if block > 0:
+                pairs += sum((cached + i) % block + 1 for i in range(new))
+                keys += min(cached + new, cached % block + new)
+            elif window > 0:
                 pairs += sum(min(window + keep_first, cached + i + 1) for i in range(new))
                 keys += min(cached + new, window + keep_first + new - 1)
             else:
@@ -1733,7 +1792,7 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         return (2.0 * pairs * n_heads * maps * (dim + vdim),
                 keys * n_kv_heads * (maps * dim + vdim) * k_cache.element_size() + t * n_heads * (4 * maps * dim + vdim * out.element_size()))
     if waves <= 0:
-        reach = ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window + keep_first)
+        reach = min(ctx.max_kv_len, block) if block > 0 else ctx.max_kv_len if window <= 0 else min(ctx.max_kv_len, window + keep_first)
         tiles = max(1, -(-reach // 64))
         waves = 1 if t * n_heads >= ATTENTION_MAPS_FULL else min(8, tiles)
     library.call("bc4g_attention_maps", _ptr(q), n_heads * maps * dim, _ptr(k_cache), _ptr(v_cache), _code(k_cache, "attention_maps"),
@@ -1741,7 +1800,7 @@ def attention_maps(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                  float(eps), float(factor), _ptr(gate), _code(gate, "attention_maps") if gate is not None else F32, gate_row, int(act),
                  _ptr(out), _code(out, "attention_maps"), t, n_heads, n_kv_heads, maps, dim, vdim, page_tokens, int(window),
                  int(keep_first), float(scale), int(waves), _ptr(sink), _ptr(far[0]) if far else None,
-                 _ptr(far[1]) if far else None, _stream(), cost=cost)
+                 _ptr(far[1]) if far else None, int(block), float(cap), _ptr(point), _stream(), cost=cost)
     return out
 
 
@@ -1851,10 +1910,13 @@ MOE_MAX_EXPERTS = 1024
 
 
 def moe_route(logits: torch.Tensor, experts: int, top: int, groups: int = 1, keep: int = 1,
-              correction: Optional[torch.Tensor] = None, want_chosen: bool = False):
+              correction: Optional[torch.Tensor] = None, want_chosen: bool = False, squash: bool = False,
+              normalize: bool = False, factor: float = 1.0):
     """The choice of experts for every row: logits float32 [T, >= experts] (the first ``experts`` columns count; rows may
     be parts of wider rows).  s = softmax(logits); the choice goes by s + correction; only experts of the ``keep`` best of
     ``groups`` equal groups of neighbours (a group counts by its largest choice) can be chosen; the ``top`` largest win.
+    ``squash``: s = sigmoid(logits), every expert by itself, instead of the softmax.  ``normalize``: the chosen experts'
+    weights are their s divided by the sum of the chosen s (+ 1e-20).  ``factor`` multiplies the weights last.
     Returns weights float32 [T, experts] -- s of the chosen, zero elsewhere -- and, if asked, the chosen int32 [T, top]."""
     _dev("moe_route", correction)
     row = _part_of_rows("moe_route", "logits", logits, experts)
@@ -1865,8 +1927,29 @@ def moe_route(logits: torch.Tensor, experts: int, top: int, groups: int = 1, kee
     weights = torch.empty((t, experts), dtype=torch.float32, device=logits.device)
     chosen = torch.empty((t, top), dtype=torch.int32, device=logits.device) if want_chosen else None
     library.call("bc4g_moe_route", _ptr(logits), row, _ptr(correction), _ptr(weights), _ptr(chosen), t, experts, groups, keep, top,
-                 _stream(), cost=lambda: (8.0 * t * experts * (1 + top), 8.0 * t * experts))
+                 1 if squash else 0, 1 if normalize else 0, float(factor), _stream(),
+                 cost=lambda: (8.0 * t * experts * (1 + top), 8.0 * t * experts))
     return (weights, chosen) if want_chosen else weights
+
+
+def routed_gelu(z: torch.Tensor, weights: Optional[torch.Tensor], experts: int, ff: int, shared_ff: int = 0,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """z [T, experts * ff + shared_ff]: every expert's ff units, then the shared unit's.  Returns (``out`` may be z itself)
+    weights[t, e] * gelu(z) with the exact gelu for expert e's units -- zero for the experts a row did not choose -- and
+    gelu(z) for the shared unit's."""
+    _dev("routed_gelu", z, weights, out)
+    t = z.shape[0]
+    if z.dim() != 2 or z.shape[1] != experts * ff + shared_ff:
+        raise KernelError(f"routed_gelu: input must be [T, {experts * ff + shared_ff}], got {tuple(z.shape)}")
+    if experts:
+        _f32("routed_gelu", "weights", weights, (t, experts))
+    if out is None:
+        out = torch.empty_like(z)
+    elif out.dtype != z.dtype or out.shape != z.shape:
+        raise KernelError("routed_gelu: out must have the input's dtype and shape")
+    library.call("bc4g_routed_gelu", _ptr(z), _ptr(out), _code(z, "routed_gelu"), _ptr(weights), t, experts, ff, shared_ff, _stream(),
+                 cost=lambda: (12.0 * z.numel(), 2 * z.numel() * z.element_size()))
+    return out
 
 
 def routed_glu(gu: torch.Tensor, weights: Optional[torch.Tensor], experts: int, ff: int, limit: float, *, shared_ff: int = 0,

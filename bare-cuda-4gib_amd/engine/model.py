@@ -38,6 +38,8 @@ class Model:
         self.embedding = _Bound(build_part("embedding", spec.embedding), spec.embedding)
         self.final_norm = _Bound(build_part("norm", spec.final_norm), spec.final_norm)
         self.head = _Bound(build_part("head", spec.head), spec.head)
+        reentry = getattr(spec, "reentry", None)
+        self.reentry = _Bound(build_part("reentry", reentry), reentry) if reentry is not None else None
         self.layers: List[Part] = []
         self._layer_bound: List[List[_Bound]] = []
         for ls in spec.layers:
@@ -59,6 +61,10 @@ class Model:
                                                        or not hasattr(self.embedding.part, "add_to")):
                 raise ConfigError("a schedule entry adds the embedding to the stream: that takes one copy of the stream and "
                                   "an embedding part that can add")
+            if getattr(e, "reenter", None) is not None and (self.reentry is None or int(getattr(spec, "streams", 1)) != 1
+                                                            or not hasattr(self.embedding.part, "beside")):
+                raise ConfigError("a schedule entry begins a pass: that takes a reentry part, one copy of the stream and an "
+                                  "embedding part that can stand beside the stream")
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
         self.max_seq_len = spec.max_seq_len
@@ -68,12 +74,13 @@ class Model:
     def all_parts(self) -> List[Part]:
         """Every part of the model, nested ones included: embedding, each layer's block with its norms,
         mixer and feed-forward, final norm, head."""
-        tops = [self.embedding.part, *self.layers, self.final_norm.part, self.head.part]
+        tops = [self.embedding.part, *([self.reentry.part] if self.reentry is not None else []), *self.layers,
+                self.final_norm.part, self.head.part]
         return [p for top in tops for p in _walk(top)]
 
     # ---- weights ------------------------------------------------------------
     def _all_bound(self) -> List[_Bound]:
-        out = [self.embedding]
+        out = [self.embedding] + ([self.reentry] if self.reentry is not None else [])
         for group in self._layer_bound:
             out.extend(group)
         out.extend([self.final_norm, self.head])
@@ -164,6 +171,10 @@ class Model:
             if e.add_embedding:
                 f, b = self.embedding.part.step_work(batch, batch.n_tokens, elem)
                 flops, nbytes = flops + f, nbytes + b
+            if getattr(e, "reenter", None) is not None:
+                for part in (self.embedding.part, self.reentry.part):
+                    f, b = part.step_work(batch, batch.n_tokens, elem)
+                    flops, nbytes = flops + f, nbytes + b
             f, b = self.layers[e.layer].step_work(batch, batch.n_tokens, elem)
             flops, nbytes = flops + f, nbytes + b
         for part in (self.final_norm.part, self.head.part):
@@ -193,10 +204,18 @@ class Model:
             layer = self.layers[e.layer]
             # (nobody prepares the first norm of an entry before which the stream changes once more)
             following = (self.layers[self.schedule[i + 1].layer]
-                         if i + 1 < len(self.schedule) and not self.schedule[i + 1].add_embedding else None)
+                         if i + 1 < len(self.schedule) and not self.schedule[i + 1].add_embedding
+                         and getattr(self.schedule[i + 1], "reenter", None) is None else None)
             ctx.handoff.begin_entry(layer, following, ctx.n_tokens)
             if e.add_embedding:
                 self.embedding.part.add_to(x, ctx)
+            if getattr(e, "reenter", None) is not None:
+                # the stream is replaced; the kernel that writes it norms it for this layer where the layer's norm can
+                first = layer.first_reader(ctx.n_tokens)[0] if hasattr(layer, "first_reader") else None
+                made = self.reentry.part.forward(x, ctx, self.embedding.part, e.reenter, first)
+                if made is not None:
+                    from ..csrc import ops
+                    ctx.handoff.leave(first, ops.Finished(made))
             layer.forward(x, ctx, ctx.cache(e.cache), e.writes)
         ctx.handoff.end_step()
         if ctx.n_logits == 0:

@@ -42,11 +42,14 @@ class ScheduleEntry:
     ``writes`` says whether this execution appends to that stream or only
     reads what another entry wrote.  ``add_embedding``: the embedding's output is added to the
     residual stream right before this execution (a stack that runs some of its layers several times
-    feeds its input in again at the start of every further pass)."""
+    feeds its input in again at the start of every further pass).  ``reenter``: the number of the pass that begins with this
+    execution -- right before it the model's ``reentry`` part replaces the stream by a map of the stream and the
+    embedding's output (None: nothing happens)."""
     layer: int
     cache: Optional[Any] = None
     writes: bool = True
     add_embedding: bool = False
+    reenter: Optional[int] = None
 
 
 @dataclasses.dataclass
@@ -62,3 +65,5 @@ class ModelSpec:
     # copies of the residual stream that the layers keep side by side, [T, streams, H] (1: the plain stream [T, H]); all
     # start as the embedding's output, and the model's last norm reads their sum
     streams: int = 1
+    # what replaces the stream before the schedule entries that say ``reenter`` (a part of category "reentry")
+    reentry: Optional[PartSpec] = None

@@ -3,26 +3,75 @@ from __future__ import annotations
 
 import torch
 
+from typing import Dict
+
+import torch
+
 from ..cache.specs import Bundle
 from ..csrc import ops
+from ..errors import ConfigError
+from ..weights.loader import WeightSpec
 from .base import Part, register_part
 from .lazy import Normed
 from .streams import StreamReader
+
+
+class LayerScale(Part):
+    """One learned number a channel by which a sublayer's output is multiplied, element by element and in float32, before it
+    joins the residual stream: x += a * f(N(x))."""
+    category = "scale"
+    graph_safe = True
+
+    def __init__(self, size: int):
+        self.size = int(size)
+        self.weight = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {"weight": WeightSpec((self.size,), kind="vector", init="ones")}
+
+    def bind(self, tensors, rt) -> None:
+        self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+    def add_to(self, x: torch.Tensor, y: torch.Tensor, next_norm=None):
+        """x += weight * y on the float32 stream; with a norm that can follow an update in the same kernel
+        (``after_update``), also that norm of the new x -- else None."""
+        if next_norm is not None and hasattr(next_norm, "after_update"):
+            return next_norm.after_update(x, y, scale=self.weight)
+        ops.stream_update(x, y, scale=self.weight)
+        return None
 
 
 class PreNormBlock(Part):
     """x += mixer(norm(x)); x += ffn(norm(x))  (reference: engine/src/model.cpp:526-604).
     The residual stream x is float32 and is updated in place.  A layer may have no feed-forward, and the mixer may read
     its input through a part that mixes every row with the row before it (``mixer_shift``, a conv part with a state of
-    its own: the layer then keeps that state beside its mixer's cache)."""
+    its own: the layer then keeps that state beside its mixer's cache).  With ``mixer_scale`` / ``ffn_scale`` (scale parts)
+    a sublayer's output is gathered in float32 and multiplied by one number a channel before it is added; the kernel
+    that adds it also norms the stream for whoever reads it next."""
     category = "block"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
-    def __init__(self, mixer, ffn, mixer_norm, ffn_norm, mixer_shift=None):
+    def __init__(self, mixer, ffn, mixer_norm, ffn_norm, mixer_shift=None, mixer_scale=None, ffn_scale=None):
         self.mixer, self.ffn, self.mixer_norm, self.ffn_norm, self.mixer_shift = mixer, ffn, mixer_norm, ffn_norm, mixer_shift
+        self.mixer_scale, self.ffn_scale = mixer_scale, ffn_scale
+        for part, scale in ((mixer, mixer_scale), (ffn, ffn_scale)):
+            if scale is not None and (part is None or not getattr(part, "adds_one_product", False)):
+                raise ConfigError("prenorm block: a scaled sublayer must give its output as one last product (adds_one_product)")
 
     def children(self):
-        return [p for p in (self.mixer_norm, self.mixer_shift, self.mixer, self.ffn_norm, self.ffn) if p is not None]
+        parts = (self.mixer_norm, self.mixer_shift, self.mixer, self.mixer_scale, self.ffn_norm, self.ffn, self.ffn_scale)
+        return [p for p in parts if p is not None]
+
+    def _scaled(self, scale, run, x, ctx) -> None:
+        """A sublayer whose output is scaled: ``run(y)`` leaves it in float32 (y an ops.Fresh), then x += scale * y, and the
+        norm of whoever reads the stream next with it."""
+        y = ops.Fresh()
+        run(y)
+        reading = ctx.handoff.reading_next
+        norm = reading[0] if reading is not None else None
+        made = scale.add_to(x, y.tensor, norm)
+        if made is not None:
+            ctx.handoff.leave(norm, ops.Finished(made))
 
     def cache_spec(self):
         """The mixer's cache, and beside it the state of the shift in front of the mixer."""
@@ -44,13 +93,21 @@ class PreNormBlock(Part):
                     h = self.mixer_shift.after(self.mixer_norm, x, ctx, cache.shift)
                 else:
                     h = self.mixer_shift.forward(self.mixer_norm.forward(x, ctx), ctx, cache.shift)
-                self.mixer.forward(h, ctx, cache.mixer, x, writes)
+                mixer_cache = cache.mixer
             else:
-                self.mixer.forward(self._normed(self.mixer, self.mixer_norm, x, ctx), ctx, cache, x, writes)
+                h, mixer_cache = self._normed(self.mixer, self.mixer_norm, x, ctx), cache
+            if self.mixer_scale is not None:
+                self._scaled(self.mixer_scale, lambda y: self.mixer.forward(h, ctx, mixer_cache, y, writes), x, ctx)
+            else:
+                self.mixer.forward(h, ctx, mixer_cache, x, writes)
         if self.ffn is None:
             return
         with handoff.reader(*(handoff.next_entry or (None, False))):
-            self.ffn.forward(self._normed(self.ffn, self.ffn_norm, x, ctx), ctx, x)
+            h = self._normed(self.ffn, self.ffn_norm, x, ctx)
+            if self.ffn_scale is not None:
+                self._scaled(self.ffn_scale, lambda y: self.ffn.forward(h, ctx, y), x, ctx)
+            else:
+                self.ffn.forward(h, ctx, x)
 
     def first_reader(self, n_rows: int):
         """(the norm this block begins with, whether its reader takes the parts of a prepared norm for a step of
@@ -179,6 +236,7 @@ class HyperBlock(Part):
             handoff.leave(following, made)
 
 
+register_part("scale", "layer_scale", LayerScale)
 register_part("block", "prenorm", PreNormBlock)
 register_part("block", "hyper", HyperBlock)
 register_part("block", "sandwich", SandwichBlock)

@@ -76,7 +76,7 @@ class TokenShift(Part):
     def after(self, norm, x: torch.Tensor, ctx, view) -> torch.Tensor:
         """The shift of norm(x) for the float32 stream x [T, H]."""
         fusable = getattr(norm, "fusable", None)
-        if fusable is None or x.dim() != 2 or x.dtype != torch.float32:
+        if fusable is None or fusable() is None or x.dim() != 2 or x.dtype != torch.float32:
             return self.forward(norm.forward(x, ctx), ctx, view)
         if self._norm is None or self._norm[0] is not norm:
             g, eps = fusable()

@@ -12,13 +12,13 @@ from .linear import linear
 
 
 class Embedding(Part):
-    """x[t, :] = float(table[ids[t], :]); no scaling, nothing added
+    """x[t, :] = float(table[ids[t], :]) * scale, nothing added; scale 1 unless a design names one
     (reference: engine/kernels/embedding_lookup.cu:16-31)."""
     category = "embedding"
     graph_safe = True     # launches kernels only: may run inside a captured graph
 
-    def __init__(self, vocab_size: int, hidden_size: int):
-        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0):
+        self.vocab_size, self.hidden_size, self.scale = int(vocab_size), int(hidden_size), float(scale)
         self.table = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -28,11 +28,15 @@ class Embedding(Part):
         self.table = tensors["weight"]
 
     def forward(self, ctx) -> torch.Tensor:
-        return ops.embed_gather(self.table, ctx.token_ids)
+        return ops.embed_gather(self.table, ctx.token_ids, factor=self.scale)
 
     def add_to(self, x: torch.Tensor, ctx) -> torch.Tensor:
         """x += the embedding of the step's tokens, in place on the float32 stream."""
-        return ops.embed_add(self.table, ctx.token_ids, x)
+        return ops.embed_add(self.table, ctx.token_ids, x, factor=self.scale)
+
+    def beside(self, x: torch.Tensor, ctx, out_dtype: torch.dtype) -> torch.Tensor:
+        """[T, 2 H] in ``out_dtype``: the stream's rows, each followed by the embedding of the row's token."""
+        return ops.embed_beside(x, self.table, ctx.token_ids, out_dtype, factor=self.scale)
 
 
 class LMHead(Part):

@@ -154,14 +154,25 @@ class RoutedExperts(Part):
     units of the experts it did not choose are multiplied by zero and those of the chosen by their weights, so that the
     second product adds up the weighted sum (the router's and the shared gate's logits are one small float32 product).
     Tensors: ``router`` [experts, hidden], ``correction`` [experts], ``e<i>.{gate,up,down}``, ``shared.{gate,up,down}``,
-    ``shared.sg`` [1, hidden]."""
+    ``shared.sg`` [1, hidden].
+
+    ``router`` "sigmoid": s = sigmoid(z), every expert by itself.  ``normalize``: the weights are the chosen experts' s divided
+    by their sum (+ 1e-20).  ``route_scale`` multiplies the weights.  ``unit`` "gelu": an expert is Wd gelu(Wu h) with the exact
+    gelu -- no gate matrix, no limit (``e<i>.{up,down}``, ``shared.{up,down}``).  ``shared_gate`` False: the shared expert is
+    added as it is (no ``shared.sg``)."""
     category = "feedforward"
     graph_safe = True     # launches kernels only: may run inside a captured graph
     accepts_lazy_norm = True
     adds_one_product = True   # the output is one last product through linear(): a block may hand it ops.Fresh
 
-    def __init__(self, hidden_size: int, experts: int, top: int, intermediate_size: int, limit: float, groups: int = 1,
-                 keep: int = 1, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0, slope: float = 1.702):
+    def __init__(self, hidden_size: int, experts: int, top: int, intermediate_size: int, limit: float = 0.0, groups: int = 1,
+                 keep: int = 1, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0, slope: float = 1.702,
+                 router: str = "softmax", normalize: bool = False, route_scale: float = 1.0, unit: str = "clamped_glu",
+                 shared_gate: bool = True):
+        if router not in ("softmax", "sigmoid") or unit not in ("clamped_glu", "gelu"):
+            raise ConfigError(f"routed experts: router {router!r} ('softmax' or 'sigmoid'), unit {unit!r} ('clamped_glu' or 'gelu')")
+        self.squash, self.normalize, self.route_scale = router == "sigmoid", bool(normalize), float(route_scale)
+        self.gated, self.shared_gate = unit == "clamped_glu", bool(shared_gate) and unit == "clamped_glu"
         self.hidden_size, self.experts, self.top, self.ff = int(hidden_size), int(experts), int(top), int(intermediate_size)
         self.limit, self.groups, self.keep, self.correction = float(limit), int(groups), int(keep), bool(correction)
         self.shared_ff, self.shared_limit, self.slope = int(shared_size), float(shared_limit), float(slope)
@@ -178,20 +189,23 @@ class RoutedExperts(Part):
         out = {"router": WeightSpec((self.experts, h))}
         if self.correction:
             out["correction"] = WeightSpec((self.experts,), kind="vector")
-        for e in range(self.experts):
-            out.update({f"e{e}.gate": WeightSpec((f, h)), f"e{e}.up": WeightSpec((f, h)), f"e{e}.down": WeightSpec((h, f))})
-        if self.shared_ff:
-            g = self.shared_ff
-            out.update({"shared.gate": WeightSpec((g, h)), "shared.up": WeightSpec((g, h)), "shared.down": WeightSpec((h, g)),
-                        "shared.sg": WeightSpec((1, h))})
+        for name, size in [(f"e{e}", f) for e in range(self.experts)] + ([("shared", self.shared_ff)] if self.shared_ff else []):
+            out.update({f"{name}.up": WeightSpec((size, h)), f"{name}.down": WeightSpec((h, size))})
+            if self.gated:
+                out[f"{name}.gate"] = WeightSpec((size, h))
+        if self.shared_ff and self.shared_gate:
+            out["shared.sg"] = WeightSpec((1, h))
         return out
 
     def bind(self, tensors, rt) -> None:
         names = [f"e{e}" for e in range(self.experts)] + (["shared"] if self.shared_ff else [])
         # per expert its gates' rows, then its ups'; the down matrices side by side along their inputs
-        self.w_gu = ops.StreamedWeight(torch.cat([tensors[f"{n}.{part}"] for n in names for part in ("gate", "up")], dim=0).contiguous())
+        # (plain units have no gates: every expert's ups' rows)
+        inner = ("gate", "up") if self.gated else ("up",)
+        self.w_gu = ops.StreamedWeight(torch.cat([tensors[f"{n}.{part}"] for n in names for part in inner], dim=0).contiguous())
         self.w_down = ops.StreamedWeight(torch.cat([tensors[f"{n}.down"] for n in names], dim=1).contiguous())
-        self.w_route = ops.StreamedWeight(torch.cat([tensors["router"]] + ([tensors["shared.sg"]] if self.shared_ff else []),
+        gated_shared = self.shared_ff and self.shared_gate
+        self.w_route = ops.StreamedWeight(torch.cat([tensors["router"]] + ([tensors["shared.sg"]] if gated_shared else []),
                                                     dim=0).contiguous())
         self.correction_w = tensors["correction"].to(torch.float32).contiguous() if self.correction else None
         self.act_dtype = rt.act_dtype
@@ -200,8 +214,9 @@ class RoutedExperts(Part):
         """What the design asks for: the router, ``top`` experts a row and the shared one; every weight read once."""
         h = self.hidden_size
         units = self.top * self.ff + self.shared_ff
-        flops = 2.0 * rows * h * (self.experts + (1 if self.shared_ff else 0)) + rows * units * (6.0 * h + 8.0)
-        nbytes = (self.experts * (3 * self.ff * h + h) + (3 * self.shared_ff * h + h if self.shared_ff else 0)) * elem
+        mats = 3 if self.gated else 2
+        flops = 2.0 * rows * h * (self.experts + (1 if self.shared_ff else 0)) + rows * units * (2.0 * mats * h + 8.0)
+        nbytes = (self.experts * (mats * self.ff * h + h) + (mats * self.shared_ff * h + h if self.shared_ff else 0)) * elem
         return flops, float(nbytes)
 
     def working_bytes_per_row(self, elem: int) -> float:
@@ -212,8 +227,12 @@ class RoutedExperts(Part):
             h = h.tensor()
         E = self.experts
         z = linear(h, self.w_route, out_dtype=torch.float32)
-        weights = ops.moe_route(z, E, self.top, self.groups, self.keep, self.correction_w)
+        weights = ops.moe_route(z, E, self.top, self.groups, self.keep, self.correction_w, squash=self.squash,
+                                normalize=self.normalize, factor=self.route_scale)
         gu = linear(h, self.w_gu, out_dtype=self.act_dtype)
+        if not self.gated:
+            linear(ops.routed_gelu(gu, weights, E, self.ff, self.shared_ff, out=gu), self.w_down, accumulate_into=residual, ctx=ctx)
+            return
         y = ops.routed_glu(gu, weights, E, self.ff, self.limit, shared_ff=self.shared_ff, shared_limit=self.shared_limit,
                            shared_logit=z[:, E:E + 1] if self.shared_ff else None, slope=self.slope)
         linear(y, self.w_down, accumulate_into=residual, ctx=ctx)

@@ -1,6 +1,7 @@
 """RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, with eps on the mean square and
 sum and rsqrt in float (reference: engine/kernels/rmsnorm.cu:16-41).  With ``offset`` the stored weight is
-counted from it: y = x * rsqrt(...) * (offset + w) -- a weight stored around zero has offset 1."""
+counted from it: y = x * rsqrt(...) * (offset + w) -- a weight stored around zero has offset 1.  With ``groups`` the row
+is cut into that many equal consecutive parts and each is divided by its own root mean square; the weight spans the row."""
 from __future__ import annotations
 
 from typing import Dict
@@ -8,6 +9,7 @@ from typing import Dict
 import torch
 
 from ..csrc import ops
+from ..errors import ConfigError
 from ..weights.loader import WeightSpec
 from .base import Part, register_part
 
@@ -16,8 +18,10 @@ class RMSNorm(Part):
     category = "norm"
     graph_safe = True
 
-    def __init__(self, size: int, eps: float, offset: float = 0.0):
-        self.size, self.eps, self.offset = int(size), float(eps), float(offset)
+    def __init__(self, size: int, eps: float, offset: float = 0.0, groups: int = 1):
+        self.size, self.eps, self.offset, self.groups = int(size), float(eps), float(offset), int(groups)
+        if self.groups <= 0 or self.size % self.groups:
+            raise ConfigError(f"rmsnorm: {self.size} channels do not fall into {self.groups} equal groups")
         self.weight = self._multiplier = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -32,16 +36,23 @@ class RMSNorm(Part):
 
     def add_to(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
         """x += norm(y), in place on the float32 residual stream: the norm after a sublayer."""
+        if self.groups != 1:
+            raise ConfigError("rmsnorm: a norm in groups is not added to the stream by a kernel of its own")
         if self._multiplier is None:
             self._multiplier = self.weight.to(torch.float32).contiguous()
         return ops.rmsnorm_add(x, y, self._multiplier, self.eps)
 
     def fusable(self):
-        """What a product needs to absorb this norm: (scale vector, eps)."""
-        return self.weight, self.eps
+        """What a product needs to absorb this norm: (scale vector, eps); None for a norm in groups, which no product absorbs."""
+        return (self.weight, self.eps) if self.groups == 1 else None
 
     def forward(self, x: torch.Tensor, ctx=None, rows=None, n_rows=None) -> torch.Tensor:
-        return ops.rmsnorm(x, self.weight, self.eps, self.out_dtype, rows=rows, n_rows=n_rows)
+        return ops.rmsnorm(x, self.weight, self.eps, self.out_dtype, rows=rows, n_rows=n_rows, groups=self.groups)
+
+    def after_update(self, x: torch.Tensor, y: torch.Tensor, scale=None, bias=None, keep: bool = True) -> torch.Tensor:
+        """x = (x if keep else 0) + scale * y + bias on the float32 stream, and this norm of the new x, in one kernel."""
+        return ops.stream_update(x, y, scale, bias, keep, norm_weight=self.weight, eps=self.eps, groups=self.groups,
+                                 out_dtype=self.out_dtype)
 
 
 class DynamicTanh(Part):

@@ -20,6 +20,10 @@ class Rotary(Part):
     cosines and sines are multiplied by 0.1 ln F + 1.  The kernels that rotate inside a product take no scaling
     (``fused()`` is None then); ``table(ctx)`` gives every row's cosines and sines to whoever rotates by a table.
 
+    A ``scaling`` that gives (factor F, original L, low, high) instead goes by a pair's wavelength l = 2 pi / inv_freq_i:
+    shorter than L / high the pair turns as it is, longer than L / low with inv_freq_i / F, and between the two with
+    (1 - s) inv_freq_i / F + s inv_freq_i, s = (L / l - low) / (high - low); cosines and sines keep their size.
+
     ``pairing`` "neighbours" turns element 2i with element 2i + 1 instead (the same angles, the same table); only
     kernels that rotate by a table know that pairing."""
     category = "position"
@@ -35,13 +39,18 @@ class Rotary(Part):
             raise ConfigError(f"rotary: theta must be positive, got {theta}")
         self.theta, self.dim = float(theta), int(dim)
         self.scaling = None
+        self.by_wavelength = False
         if scaling is not None:
+            self.by_wavelength = isinstance(scaling, dict) and "low" in scaling and "high" in scaling
+            keys = ("factor", "original", "low", "high") if self.by_wavelength else ("factor", "original", "fast", "slow")
             try:
-                self.scaling = tuple(float(scaling[k]) for k in ("factor", "original", "fast", "slow"))
+                self.scaling = tuple(float(scaling[k]) for k in keys)
             except (KeyError, TypeError, ValueError):
-                raise ConfigError(f"rotary: scaling must give factor, original, fast and slow, got {scaling!r}") from None
-            if min(self.scaling) <= 0 or self.theta == 1.0:
+                raise ConfigError(f"rotary: scaling must give {', '.join(keys)}, got {scaling!r}") from None
+            if min(self.scaling) <= 0 or (self.theta == 1.0 and not self.by_wavelength):
                 raise ConfigError(f"rotary: scaling {scaling!r} with theta {theta}: every number must be positive, theta not 1")
+            if self.by_wavelength and self.scaling[2] == self.scaling[3]:
+                raise ConfigError(f"rotary: scaling {scaling!r}: low and high must differ")
         self._freqs = None
 
     def fused(self):
@@ -61,6 +70,18 @@ class Rotary(Part):
         freqs = [self.theta ** (-2.0 * i / self.dim) for i in range(half)]
         if self.scaling is None:
             return freqs, 1.0
+        if self.by_wavelength:
+            factor, original, low, high = self.scaling
+            out = []
+            for f in freqs:
+                wavelength = 2.0 * math.pi / f
+                if wavelength > original / low:
+                    f = f / factor
+                elif wavelength >= original / high:
+                    s = (original / wavelength - low) / (high - low)
+                    f = (1.0 - s) * f / factor + s * f
+                out.append(f)
+            return out, 1.0
         factor, original, fast, slow = self.scaling
         where = lambda t: self.dim * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))      # noqa: E731
         lo, hi = max(math.floor(where(fast)), 0), min(math.ceil(where(slow)), self.dim - 1)
@@ -74,7 +95,7 @@ class Rotary(Part):
         freqs, amplitude = self.frequencies()
         if self._freqs is None or self._freqs.device != ctx.positions.device:
             self._freqs = torch.tensor(freqs, dtype=torch.float64, device=ctx.positions.device)
-        return ctx.shared(("rotary_table", self.dim, self.theta, self.scaling),
+        return ctx.shared(("rotary_table", self.dim, self.theta, self.scaling, self.by_wavelength),
                           lambda: ops.rotary_table(ctx.positions, self._freqs, amplitude))
 
 
