@@ -94,8 +94,13 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Ten
         out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
     elif out.dtype != torch.float32 or tuple(out.shape) != (n, hidden):
         raise KernelError(f"embed_gather: out must be float32 [{n}, {hidden}]")
-    library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out),
-                 n, hidden, vocab, float(factor), 0, _stream(), cost=lambda: (0.0, n * hidden * (table.element_size() + 4)))
+    cost = lambda: (0.0, n * hidden * (table.element_size() + 4))      # noqa: E731
+    if factor == 1.0:
+        library.call("bc4g_embed_gather", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out), n, hidden, vocab, _stream(),
+                     cost=cost)
+    else:
+        library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_gather"), _ptr(ids), _ptr(out), n, hidden, vocab, float(factor),
+                     0, _stream(), cost=cost)
     return out
 
 
@@ -107,8 +112,12 @@ def embed_add(table: torch.Tensor, ids: torch.Tensor, x: torch.Tensor, factor: f
     _i32("embed_add", "ids", ids, n)
     if x.dtype != torch.float32 or tuple(x.shape) != (n, hidden) or not x.is_contiguous():
         raise KernelError(f"embed_add: x must be float32 [{n}, {hidden}], got {x.dtype} {tuple(x.shape)}")
-    library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, float(factor), 1,
-                 _stream(), cost=lambda: (1.0 * n * hidden, n * hidden * (table.element_size() + 8)))
+    cost = lambda: (1.0 * n * hidden, n * hidden * (table.element_size() + 8))      # noqa: E731
+    if factor == 1.0:
+        library.call("bc4g_embed_add", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, _stream(), cost=cost)
+    else:
+        library.call("bc4g_embed_rows", _ptr(table), _code(table, "embed_add"), _ptr(ids), _ptr(x), n, hidden, vocab, float(factor), 1,
+                     _stream(), cost=cost)
     return x
 
 
@@ -174,9 +183,13 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     if groups <= 0 or hidden % groups:
         raise KernelError(f"rmsnorm: {hidden} channels do not fall into {groups} equal groups")
     out = torch.empty((n, hidden), dtype=out_dtype, device=x.device)
-    library.call("bc4g_rmsnorm_groups", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
-                 _code(out, "rmsnorm"), n, hidden, int(groups), float(eps), _stream(),
-                 cost=lambda: (3.0 * n * hidden, n * hidden * (4 + out.element_size()) + hidden * weight.element_size()))
+    cost = lambda: (3.0 * n * hidden, n * hidden * (4 + out.element_size()) + hidden * weight.element_size())      # noqa: E731
+    if groups == 1:
+        library.call("bc4g_rmsnorm", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
+                     _code(out, "rmsnorm"), n, hidden, float(eps), _stream(), cost=cost)
+    else:
+        library.call("bc4g_rmsnorm_groups", _ptr(x), _ptr(rows), _ptr(weight), _code(weight, "rmsnorm"), _ptr(out),
+                     _code(out, "rmsnorm"), n, hidden, int(groups), float(eps), _stream(), cost=cost)
     return out
 
 

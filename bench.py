@@ -123,6 +123,32 @@ MILENEX_SIZES = {
     "2k": (milenex_shape(2048, 5, 16, 4, 64, 128, 8192, 8, 2, 1792), NAGEZEN_SIZES["2k"][0]),
     "4k": (milenex_shape(4096, 5, 32, 8, 64, 128, 14336, 8, 2, 3200), NAGEZEN_SIZES["4k"][0]),
 }
+
+
+def lagusun_shape(width, layers, heads, kv_heads, dim, vdim, experts, top, expert_ff, span=1024, vocab=32000):
+    """A Lagusun configuration of real layer sizes: attention by blocks whose values are its keys and windowed attention
+    with sigmoid weights in turn; every feed-forward ``top`` of ``experts`` routed gelu experts with a shared one; norms in
+    two groups; the second layer runs twice, the stream being replaced before each of its passes."""
+    moe = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top, scale=2.0), shared=dict(ff=expert_ff))
+    one = dict(type="attention", mixer=dict(heads=heads, kv_heads=kv_heads, dim=vdim, vdim=vdim, scale=vdim ** -0.5,
+                                            mask=dict(size=span), rot=dict(base=10000.0, dims=vdim // 2)))
+    two = dict(type="attention_2", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, softcap=30.0,
+                                              mask=dict(size=span),
+                                              rot=dict(base=10000.0, dims=dim, scaling=dict(factor=8.0, low=1.0, high=4.0, original=2048))))
+    order = [dict(one if i % 2 == 0 else two, mlp=moe) for i in range(layers)]
+    return dict(architecture="Lagusun", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=2), embedding=dict(scale=float(width) ** 0.5),
+                loop=dict(start=1, stop=2, times=2), layers=order)
+
+
+# --only lagusun: the design at a few sizes that resemble a real model's layers (five layers, six layer runs; a row uses
+# two of eight experts and the shared one; an expert's two matrices hold what a Milenex expert's three do), each beside
+# the Milenex decoder (the other design here with windowed float32 attention, routed experts and layers that run twice)
+# of the same width, number of layer runs and head count.
+LAGUSUN_SIZES = {
+    "1k": (lagusun_shape(1024, 5, 8, 2, 64, 128, 8, 2, 1344), MILENEX_SIZES["1k"][0]),
+    "2k": (lagusun_shape(2048, 5, 16, 4, 64, 128, 8, 2, 2688), MILENEX_SIZES["2k"][0]),
+    "4k": (lagusun_shape(4096, 5, 32, 8, 64, 128, 8, 2, 4800), MILENEX_SIZES["4k"][0]),
+}
 BASELINE_DECODE_B1 = 77.3                   # the reference's only FP16 decode number (batch 1, RTX 3050)
 
 
@@ -295,7 +321,7 @@ def kernel_table(model, cfg, prefill_tokens, batch, context, dtype):
 
 def run_mamenex(size, args, only="mamenex", names=("mamenex", "llama"), sizes=None):
     """Prefill and decode of a design at one size beside another decoder of equal size (Mamenex beside Llama, Nagezen
-    beside Mamenex, Milenex beside Nagezen); with --kernels the per-kernel tables of both."""
+    beside Mamenex, Milenex beside Nagezen, Lagusun beside Milenex); with --kernels the per-kernel tables of both."""
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     elem = 2 if args.dtype == "bf16" else 4
     line = {"only": only, "size": size, "dtype": args.dtype, "prefill_tokens": args.prefill_tokens, "batch": args.batch,
@@ -463,9 +489,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0, help="--only serve: ... and this top-p (1: none)")
     ap.add_argument("--gather-ms", type=float, default=0.0,
                     help="--only chat: the scheduler waits this long before it admits those who came while others decode")
-    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex, nagezen, milenex: which of the sizes " + ", ".join(MAMENEX_SIZES))
-    ap.add_argument("--kernels", action="store_true", help="--only mamenex, nagezen, milenex: add the per-kernel tables (time, part of the roofline)")
-    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex", "nagezen", "milenex"], default=None,
+    ap.add_argument("--sizes", default="1k,2k,4k", help="--only mamenex, nagezen, milenex, lagusun: which of the sizes " + ", ".join(MAMENEX_SIZES))
+    ap.add_argument("--kernels", action="store_true", help="--only mamenex, nagezen, milenex, lagusun: add the per-kernel tables (time, part of the roofline)")
+    ap.add_argument("--only", choices=["decode", "prefill", "serve", "chat", "gemm", "peaks", "mamenex", "nagezen", "milenex", "lagusun"], default=None,
                     help="run one part only and print its own short line (for profiling); peaks: what a kernel that only "
                          "reads, and one of nothing but matrix-core instructions, reach on this device")
     ap.add_argument("--mnk", default="2048,11264,2048",
@@ -493,6 +519,10 @@ def main() -> int:
     if args.only == "milenex":
         for size in args.sizes.split(","):
             print(json.dumps(run_mamenex(size, args, "milenex", ("milenex", "nagezen"), MILENEX_SIZES)), flush=True)
+        return 0
+    if args.only == "lagusun":
+        for size in args.sizes.split(","):
+            print(json.dumps(run_mamenex(size, args, "lagusun", ("lagusun", "milenex"), LAGUSUN_SIZES)), flush=True)
         return 0
     from bare_cuda_4gib_amd.csrc.peaks import measured_peaks
     measured = measured_peaks()
