@@ -76,10 +76,32 @@ __global__ __launch_bounds__(kWave) void heads_prepare_kernel(const PrepareSecti
   if (norm_w && p.norm_rows) {      // the mean square of the whole row, all heads at once; the weight spans the row too
     const int width = p.heads * dim;
     float all = 0.f;
-    for (int c = lane; c < width; c += kWave) {
-      float v = load_any(p.in, p.in_dtype, row * p.in_row + c);
-      if (bias) v += bias[c];
-      all = fmaf(v, v, all);
+    const bf16_t* row16 = static_cast<const bf16_t*>(p.in) + row * p.in_row;
+    const float* row32 = static_cast<const float*>(p.in) + row * p.in_row;
+    // (which way the sum is taken depends on the section alone, never on the row: every row's base is aligned or none is)
+    const bool aligned = reinterpret_cast<uintptr_t>(p.in) % 16 == 0 && p.in_row % 8 == 0;
+    if (!bias && p.in_dtype == kBF16 && width % 8 == 0 && aligned) {
+      // every wave of the row reads the whole row for this sum: in 16-byte pieces, eight elements a lane
+      for (int c = lane * 8; c < width; c += kWave * 8) {
+        const uint4 bits = *reinterpret_cast<const uint4*>(row16 + c);
+        const uint32_t w4[4] = {bits.x, bits.y, bits.z, bits.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float lo = __uint_as_float(w4[e] << 16), hi = __uint_as_float(w4[e] & 0xffff0000u);
+          all = fmaf(lo, lo, all), all = fmaf(hi, hi, all);
+        }
+      }
+    } else if (!bias && p.in_dtype == kF32 && width % 4 == 0 && aligned) {
+      for (int c = lane * 4; c < width; c += kWave * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(row32 + c);
+        all = fmaf(v.x, v.x, all), all = fmaf(v.y, v.y, all), all = fmaf(v.z, v.z, all), all = fmaf(v.w, v.w, all);
+      }
+    } else {
+      for (int c = lane; c < width; c += kWave) {
+        float v = load_any(p.in, p.in_dtype, row * p.in_row + c);
+        if (bias) v += bias[c];
+        all = fmaf(v, v, all);
+      }
     }
     scale = 1.0f / sqrtf(wave_sum(all) / static_cast<float>(width) + p.eps);
     norm_w += static_cast<long>(head) * dim;

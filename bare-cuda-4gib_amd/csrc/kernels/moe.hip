@@ -104,16 +104,25 @@ __global__ __launch_bounds__(kWave) void moe_route_kernel(const float* __restric
 
 __device__ inline float gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
-template <typename T>
-__global__ void routed_gelu_kernel(const T* __restrict__ z, T* __restrict__ out, const float* __restrict__ weights, long total,
+// PIECE elements a thread (16 bytes), all of one expert: ff and shared_ff are multiples of PIECE (1: any sizes).
+template <typename T, int PIECE>
+__global__ void routed_gelu_kernel(const T* z, T* out, const float* __restrict__ weights, long total,      // (out may be z)
                                    int experts, int ff, int shared_ff) {
   const int row_width = experts * ff + shared_ff;
-  const long stride = static_cast<long>(blockDim.x) * gridDim.x;
-  for (long i = blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x; i < total; i += stride) {
+  const long stride = static_cast<long>(blockDim.x) * gridDim.x * PIECE;
+  for (long i = (blockIdx.x * static_cast<long>(blockDim.x) + threadIdx.x) * PIECE; i < total; i += stride) {
     const long r = i / row_width;
     const int c = static_cast<int>(i - r * row_width);
     const float w = c < experts * ff ? weights[r * experts + c / ff] : 1.0f;
-    out[i] = from_float<T>(w != 0.f ? w * gelu_erf(to_float(z[i])) : 0.f);
+    if (PIECE == 1) {
+      out[i] = from_float<T>(w != 0.f ? w * gelu_erf(to_float(z[i])) : 0.f);
+    } else {
+      __align__(16) T piece[PIECE];
+      *reinterpret_cast<uint4*>(piece) = w != 0.f ? *reinterpret_cast<const uint4*>(z + i) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int e = 0; e < PIECE; ++e) piece[e] = from_float<T>(w != 0.f ? w * gelu_erf(to_float(piece[e])) : 0.f);
+      *reinterpret_cast<uint4*>(out + i) = *reinterpret_cast<const uint4*>(piece);
+    }
   }
 }
 
@@ -177,16 +186,22 @@ extern "C" int bc4g_routed_gelu(const void* z, void* out, int dtype, const float
   const long total = static_cast<long>(n_rows) * (static_cast<long>(experts) * ff + shared_ff);
   if (total == 0) return 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const long blocks = (total + kBlock - 1) / kBlock;
+  const int piece = dtype == kF32 ? 4 : 8;      // elements in 16 bytes
+  const bool pieces = ff % piece == 0 && shared_ff % piece == 0 && reinterpret_cast<uintptr_t>(z) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const long threads = pieces ? total / piece : total;
+  const long blocks = (threads + kBlock - 1) / kBlock;
   const int grid = static_cast<int>(blocks > 65535 ? 65535 : blocks);
-  if (dtype == kF32)
-    routed_gelu_kernel<float><<<grid, kBlock, 0, s>>>(static_cast<const float*>(z), static_cast<float*>(out), weights, total,
-                                                      experts, ff, shared_ff);
-  else if (dtype == kBF16)
-    routed_gelu_kernel<bf16_t><<<grid, kBlock, 0, s>>>(static_cast<const bf16_t*>(z), static_cast<bf16_t*>(out), weights, total,
-                                                       experts, ff, shared_ff);
-  else
+#define BC4G_ROUTED_GELU(T, P)                                                                                              \
+  routed_gelu_kernel<T, P><<<grid, kBlock, 0, s>>>(static_cast<const T*>(z), static_cast<T*>(out), weights, total, experts, ff, shared_ff)
+  if (dtype == kF32) {
+    if (pieces) BC4G_ROUTED_GELU(float, 4); else BC4G_ROUTED_GELU(float, 1);
+  } else if (dtype == kBF16) {
+    if (pieces) BC4G_ROUTED_GELU(bf16_t, 8); else BC4G_ROUTED_GELU(bf16_t, 1);
+  } else {
     return fail("routed_gelu: unknown dtype %d", dtype);
+  }
+#undef BC4G_ROUTED_GELU
   return check_launch("routed_gelu");
 }
 
