@@ -44,6 +44,12 @@ bool embed() {
     for (int r = 0; r < n; ++r)
       for (int c = 0; c < hidden; ++c) want.push_back(source[static_cast<size_t>(ids[r]) * hidden + c]);
     ok &= close(dtype ? "rows of a bfloat16 table" : "rows of a float table", widen(out.get()), want, 0.0, 0.0);
+    // the same rows times a factor, stored and then added to what is there
+    const float factor = 2.5f;
+    RUN(bc4g_embed_rows(dtype ? static_cast<const void*>(t16.p) : t32.p, dtype, di.p, out.p, n, hidden, vocab, factor, 0, kStream));
+    RUN(bc4g_embed_rows(dtype ? static_cast<const void*>(t16.p) : t32.p, dtype, di.p, out.p, n, hidden, vocab, factor, 1, kStream));
+    for (double& v : want) v *= 2.0 * factor;
+    ok &= close(dtype ? "scaled rows of a bfloat16 table" : "scaled rows of a float table", widen(out.get()), want, 1e-6, 0.0);
   }
   return ok;
 }
@@ -75,6 +81,18 @@ bool rmsnorm() {
       }
       const std::vector<double> got = out_dtype ? widen(o16.get()) : widen(o32.get());
       ok &= close("gathered rows", got, want, out_dtype ? kBf16 : 1e-5, 1e-6);
+      // the same rows in four parts of ten, each divided by its own root mean square
+      const int groups = 4, part = hidden / groups;
+      RUN(bc4g_rmsnorm_groups(dx.p, dr.p, w_dtype ? static_cast<const void*>(w16.p) : w32.p, w_dtype,
+                              out_dtype ? static_cast<void*>(o16.p) : o32.p, out_dtype, m, hidden, groups, eps, kStream));
+      std::vector<double> parts;
+      for (int r = 0; r < m; ++r)
+        for (int g = 0; g < groups; ++g) {
+          const std::vector<double> y = plain::rmsnorm(take(widen(x), static_cast<size_t>(rows[r]) * hidden + g * part, part),
+                                                       take(scale, static_cast<size_t>(g) * part, part), eps);
+          parts.insert(parts.end(), y.begin(), y.end());
+        }
+      ok &= close("gathered rows in groups", out_dtype ? widen(o16.get()) : widen(o32.get()), parts, out_dtype ? kBf16 : 1e-5, 1e-6);
     }
   return ok;
 }

@@ -129,12 +129,12 @@ def lagusun_shape(width, layers, heads, kv_heads, dim, vdim, experts, top, exper
     """A Lagusun configuration of real layer sizes: attention by blocks whose values are its keys and windowed attention
     with sigmoid weights in turn; every feed-forward ``top`` of ``experts`` routed gelu experts with a shared one; norms in
     two groups; the second layer runs twice, the stream being replaced before each of its passes."""
-    moe = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top, scale=2.0), shared=dict(ff=expert_ff))
+    moe = dict(kind="moe", expert=dict(ff=expert_ff), router=dict(experts=experts, top=top, scale=1.5), shared=dict(ff=expert_ff))
     one = dict(type="attention", mixer=dict(heads=heads, kv_heads=kv_heads, dim=vdim, vdim=vdim, scale=vdim ** -0.5,
                                             mask=dict(size=span), rot=dict(base=10000.0, dims=vdim // 2)))
     two = dict(type="attention_2", mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, softcap=30.0,
                                               mask=dict(size=span),
-                                              rot=dict(base=10000.0, dims=dim, scaling=dict(factor=8.0, low=1.0, high=4.0, original=2048))))
+                                              rot=dict(base=10000.0, dims=dim, scaling=dict(factor=4.0, low=1.0, high=2.0, original=2048))))
     order = [dict(one if i % 2 == 0 else two, mlp=moe) for i in range(layers)]
     return dict(architecture="Lagusun", vocab=vocab, width=width, norm=dict(eps=1e-6, groups=2), embedding=dict(scale=float(width) ** 0.5),
                 loop=dict(start=1, stop=2, times=2), layers=order)

@@ -62,7 +62,7 @@ CONFIGS: Dict[str, dict] = {
         attention_2(6, 2, 8, 12, window=20, dims=4, base=30.0, softcap=30.0, scale=0.6, mlp=None),
         attention(2, 1, 16, block=33, dims=16, base=50.0, mlp=moe(5, 5, 12, scale=0.5, shared=9))]),
     "B": dict(architecture="Lagusun", vocab=131, width=64, norm=dict(eps=1e-6, groups=1), layers=[
-        attention_2(6, 1, 24, 130, window=50, dims=12, base=1000.0, scaling=(8.0, 1.0, 4.0, 64), mlp=moe(3, 2, 40, shared=24)),
+        attention_2(6, 1, 24, 130, window=50, dims=12, base=1000.0, scaling=(6.0, 1.0, 3.0, 64), mlp=moe(3, 2, 40, shared=24)),
         attention(2, 2, 40, block=70, dims=24, mlp=None),
         attention(3, 1, 72, block=17, dims=72, base=1000.0, scale=0.2, mlp=moe(8, 3, 16, scale=2.5))]),
     "C": dict(architecture="Lagusun", vocab=77, width=42, norm=dict(eps=1e-3, groups=2), embedding=dict(scale=0.7),
@@ -86,8 +86,14 @@ CONFIGS: Dict[str, dict] = {
     "F": dict(architecture="Lagusun", vocab=40, width=20, norm=dict(eps=1e-4, groups=5), loop=dict(start=1, stop=2, times=1), layers=[
         attention_2(2, 1, 6, 10, window=2, dims=6, base=9.0, mlp=moe(3, 1, 6, shared=4)),
         attention(2, 1, 10, block=100, dims=10, base=9.0, mlp=moe(4, 2, 6))]),
+    # widths at which the products take their matrix-core forms: multiples of 64 throughout, a prompt of a few hundred rows
+    "G": dict(architecture="Lagusun", vocab=300, width=192, norm=dict(eps=1e-5, groups=2), embedding=dict(scale=8.0),
+              loop=dict(start=0, stop=2, times=2), layers=[
+        attention(6, 3, 32, block=48, dims=16, base=5000.0, mlp=moe(4, 2, 128, scale=1.5, shared=64)),
+        attention_2(4, 2, 48, 64, window=40, dims=32, base=5000.0, scaling=(4.0, 1.0, 2.0, 128), softcap=20.0, mlp=moe(8, 2, 64, shared=128)),
+        attention_2(8, 8, 16, 16, window=130, dims=16, softcap=10.0, mlp=moe(4, 3, 64))]),
 }
-SEEDS = {"A": 13, "B": 24, "C": 35, "D": 46, "E": 57, "F": 68}
+SEEDS = {"A": 13, "B": 24, "C": 35, "D": 46, "E": 57, "F": 68, "G": 79}
 
 
 def every_expert(config: dict) -> dict:

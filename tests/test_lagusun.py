@@ -111,8 +111,8 @@ def test_absent_keys_have_the_design_s_defaults():
     assert model.layers[2].ffn.route_scale == 2.5 and model.layers[1].ffn is None
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(10, 100.0, (4.0, 1.0, 3.0, 40)), (12, 1000.0, (8.0, 1.0, 4.0, 64)), (6, 20.0, (2.0, 0.5, 2.0, 16)),
-                                               (8, 300.0, (16.0, 2.0, 8.0, 100)), (64, 500000.0, (8.0, 1.0, 4.0, 8192)), (6, 9.0, None)])
+@pytest.mark.parametrize("dims,base,scaling", [(10, 100.0, (4.0, 1.0, 3.0, 40)), (12, 1000.0, (6.0, 1.0, 3.0, 64)), (6, 20.0, (2.0, 0.5, 2.0, 16)),
+                                               (8, 300.0, (16.0, 2.0, 8.0, 100)), (64, 250000.0, (6.0, 1.0, 3.0, 4096)), (6, 9.0, None)])
 def test_the_rotary_part_scales_frequencies_by_wavelength(dims, base, scaling):
     from bare_cuda_4gib_amd.parts.position import Rotary
     as_dict = dict(zip(("factor", "low", "high", "original"), scaling)) if scaling else None
@@ -173,3 +173,18 @@ def test_the_plain_model_does_not_look_ahead_and_every_piece_counts(name, tmp_pa
         model.w[key] = kept * 1.1
         assert float((model.forward(ids) - whole).abs().max()) > 1e-3, key
         model.w[key] = kept
+
+
+def test_the_random_weights_mode_writes_a_folder_that_loads(tmp_path):
+    """The framework's own random-weights mode over a Lagusun configuration: every tensor the design names, norm weights
+    and the sublayers' scales at one, a folder whose configuration reads back."""
+    from bare_cuda_4gib_amd.config.registry import load_config
+    from bare_cuda_4gib_amd.weights import write_random_model
+    from safetensors.torch import load_file
+    folder = write_random_model(lagusun_models.CONFIGS["A"], 5, str(tmp_path / "random"), "bfloat16")
+    arch, cfg = load_config(folder)
+    assert arch.name == "Lagusun" and cfg.embedding_scale == 2.5 and cfg.norm_groups == 3
+    tensors = load_file(folder + "/model.safetensors")
+    assert set(tensors) == set(lagusun_models.tensors_for(lagusun_models.CONFIGS["A"], 1))
+    assert bool((tensors["l1.ls1"] == 1.0).all()) and bool((tensors["l0.norm2"] == 1.0).all())
+    assert tuple(tensors["loop.step"].shape) == (2, 48) and float(tensors["loop.in"].float().std()) > 0

@@ -25,7 +25,7 @@ pytestmark = pytest.mark.gpu
 # mean square over the vocabulary), and no single logit by more than ten times that.
 ROW_RMS = {"float32": 2e-5, "bfloat16": 6e-2}
 LENGTHS = {"A": [1, 2, 9, 70, 150], "B": [3, 33, 64, 141], "C": [1, 17, 140], "D": [2, 66, 131, 200], "E": [1, 2, 3, 65, 190],
-           "F": [1, 5, 101, 130]}
+           "F": [1, 5, 101, 130], "G": [5, 150, 260]}
 CLOSE_CALL = 1e-5       # a 32-bit run is held to the plain rows up to a request's first routing margin below this
 DEV = "cuda:0"
 
@@ -99,7 +99,7 @@ CASES = [(n, d) for n in sorted(lagusun_models.CONFIGS) for d in ("float32", "bf
 def test_whole_prompts(setups, name, dtype):
     folder, requests, logits, upto = setups(name, dtype)
     steps, where = helpers.trace_whole(requests)
-    got = helpers.replay_in_process(executor(folder, dtype, 20, 16), steps)
+    got = helpers.replay_in_process(executor(folder, dtype, 40, 16), steps)
     close_rows(got, where, logits, dtype, f"whole {name} {dtype}", upto=upto)
 
 
@@ -160,7 +160,7 @@ def test_mixed_batches_with_pages_and_slots_used_again(setups, name, dtype):
     plain_logits.update({rid + "again": logits[rid] for rid in requests})
     for seed in (3, 4):
         steps, where, peak = helpers.trace_mixed(many, seed, max_live=3, tail=10, page_tokens=16)
-        ex = executor(folder, dtype, peak // 16, 16, max_requests=3, max_tokens=208)
+        ex = executor(folder, dtype, peak // 16, 16, max_requests=3, max_tokens=272)
         got = helpers.replay_in_process(ex, steps)
         close_rows(got, where, plain_logits, dtype, f"mixed {name} {dtype} {seed}", upto=upto)
         assert ex.cache.pages_in_use() == 0 and ex.cache.free_slots == 3
@@ -360,7 +360,7 @@ def rotary_table(positions, dims, base, scaling):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads,dim,dims,base,scaling", [(3, 8, 8, 10000.0, None), (2, 48, 24, 500.0, (8.0, 1.0, 4.0, 64)),
+@pytest.mark.parametrize("heads,dim,dims,base,scaling", [(3, 8, 8, 10000.0, None), (2, 48, 24, 500.0, (6.0, 1.0, 3.0, 64)),
                                                          (5, 7, 6, 30.0, (2.0, 0.5, 2.0, 16)), (1, 130, 2, 7.0, None), (4, 10, 0, 1.0, None)])
 def test_queries_and_keys_normed_over_the_whole_projection_then_rotated(dtype, heads, dim, dims, base, scaling):
     """The norm runs over all heads at once with a weight that spans them (one head made large shrinks the others), then
@@ -402,7 +402,7 @@ def test_a_bias_then_the_rotation_then_the_unit_norm_a_head(dtype, heads, dim, d
     T, eps = 5, 1e-2
     x, b = (torch.randn(T, heads * dim) * 0.2).to(dtype), torch.randn(heads * dim) * 0.2
     positions = torch.tensor([0, 1, 33, 1000, 70001], dtype=torch.int32)
-    scaling = dict(factor=8.0, low=1.0, high=4.0, original=64)
+    scaling = dict(factor=5.0, low=1.0, high=3.0, original=64)
     table = rotary_table(positions, dims, 50.0, scaling) if dims else None
     freqs = plain.scaled_frequencies(dims, 50.0, scaling)
     want = plain.unit_rms(plain.half_rotation((x.double() + b.double()).view(T, heads, dim), positions, freqs), eps)
