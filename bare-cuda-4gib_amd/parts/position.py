@@ -20,9 +20,9 @@ class Rotary(Part):
     cosines and sines are multiplied by 0.1 ln F + 1.  The kernels that rotate inside a product take no scaling
     (``fused()`` is None then); ``table(ctx)`` gives every row's cosines and sines to whoever rotates by a table.
 
-    A ``scaling`` that gives (factor F, original L, low, high) instead goes by a pair's wavelength l = 2 pi / inv_freq_i:
-    shorter than L / high the pair turns as it is, longer than L / low with inv_freq_i / F, and between the two with
-    (1 - s) inv_freq_i / F + s inv_freq_i, s = (L / l - low) / (high - low); cosines and sines keep their size.
+    A ``scaling`` that gives (factor F, original L, low, high) instead goes by r_i = L inv_freq_i / (2 pi), the turns a pair
+    makes over L positions: above ``high`` the pair turns as it is, below ``low`` with inv_freq_i / F, and from low to high with
+    inv_freq_i (s + (1 - s) / F), s = (r_i - low) / (high - low); cosines and sines keep their size.
 
     ``pairing`` "neighbours" turns element 2i with element 2i + 1 instead (the same angles, the same table); only
     kernels that rotate by a table know that pairing."""

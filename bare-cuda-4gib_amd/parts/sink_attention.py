@@ -35,7 +35,7 @@ class SinkAttention(Part):
     Further parameters, each alone or with the others (not with mixed weights or a head gate):
 
     bias        ``q.b``, ``k.b``, ``v.b`` are added to the projections
-    values      "keys": there is no Wv -- the values are the keys as projected (before any norm or rotation), vdim = dim
+    values      "keys": there is no Wv -- a value head is its key head straight out of the product (what the keys go through afterwards does not touch it), vdim = dim
     row_norm    q and k are normed over their whole projection, all heads at once, each with a weight that spans it
                 (``q.norm`` [heads * dim], ``k.norm`` [kv_heads * dim]), before the rotation
     value_unit_norm  every value head divided by sqrt(mean(head^2) + eps), no weight; cached so
@@ -60,7 +60,7 @@ class SinkAttention(Part):
             raise ConfigError(f"sink attention: block {block} and cap {cap} must not be negative, and a block mask stands "
                               f"instead of a window ({window})")
         if values == "keys" and (dim != vdim or conv_taps):
-            raise ConfigError(f"sink attention: values that are the keys as projected have the keys' size ({dim}, not {vdim}) "
+            raise ConfigError(f"sink attention: values taken from the key product have the keys' size ({dim}, not {vdim}) "
                               "and no convolution behind the projections")
         if heads <= 0 or kv_heads <= 0 or heads % kv_heads:
             raise ConfigError(f"sink attention: {heads} heads cannot share {kv_heads} key/value heads")
@@ -188,7 +188,7 @@ class SinkAttention(Part):
             kv = cache.kv if self.conv_taps > 1 else cache
             qkv = ops.causal_conv(x[:, :self.channels] if self.head_gate else x, self.conv_w, tail, ctx)
         q, k = qkv[:, :nq], qkv[:, nq:nq + nk]
-        v = qkv[:, nq + nk:nq + nk + nv] if self.own_values else k      # (else the keys as projected)
+        v = qkv[:, nq + nk:nq + nk + nv] if self.own_values else k      # (else the key product's columns, untouched)
         table = self.position.table(ctx) if self.position is not None else None
         turn = dict(table=table, neighbours=bool(getattr(self.position, "neighbours", False)), unit_after=self.unit_norm, eps=self.eps,
                     norm_rows=self.row_norm)

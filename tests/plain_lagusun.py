@@ -13,10 +13,10 @@ sequence's tokens from 0):
   N(v)       v cut into n equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps), the whole times g
   loop       layers a..b-1 run n times in a row with the same weights (each pass with a cache of its own); right before
              the first layer of pass t (t = 0 too)  x = W_in [x; x0] + s_t
-  rotation   the first ``dims`` elements of a head, element i with element i + dims/2; the pair (u, v) at position p
-             becomes (u cos a - v sin a, v cos a + u sin a), a = p f_i, f_i = base^(-2i/dims); with ``scaling`` the
-             slow frequencies are divided by a factor, the fast ones kept, those between blended
-  mixers     ``attention``    q = Wq h, k = Wk h, values = the keys as projected; q and k each normed over the whole
+  rotation   of a head's first ``dims`` elements, in two halves: (lo_i, hi_i) = (element i, element i + dims/2) turns by the
+             angle t = p w_i at position p, w_i = base^(-2i/dims): lo' = lo cos t - hi sin t, hi' = hi cos t + lo sin t;
+             with ``scaling`` the slow w_i are divided by a factor, the fast ones kept, those between blended
+  mixers     ``attention``    q = Wq h, k = Wk h, values = k straight out of its product; q and k each normed over the whole
                               projection (all heads at once, with a weight), then rotated; a row sees the keys of its
                               own block of ``mask.size`` positions up to itself; softmax with one more term, exp(0),
                               in the denominator
@@ -53,9 +53,9 @@ def grouped_norm(v: torch.Tensor, g: torch.Tensor, eps: float, groups: int) -> t
 
 
 def scaled_frequencies(dims: int, base: float, scaling: Optional[dict]) -> torch.Tensor:
-    """f_i = base^(-2i/dims) for i < dims/2; with ``scaling`` (factor, low, high, original) by wavelength l = 2 pi / f:
-    shorter than original/high: f; longer than original/low: f / factor; between: the blend
-    (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
+    """w_i = base^(-2i/dims) for i < dims/2.  With ``scaling`` (factor F, low, high, original L) a pair is judged by
+    r = L w / (2 pi), the turns it makes over L positions: r > high leaves w, r < low gives w / F, and from low to high
+    w (s + (1 - s) / F) with s = (r - low) / (high - low)."""
     out = []
     for i in range(dims // 2):
         f = base ** (-2.0 * i / dims)
@@ -181,7 +181,7 @@ class PlainLagusun:
         w, T = self.w, h.shape[0]
         H, G, d = m["heads"], m["kv_heads"], m["dim"]
         q, k = h @ w[p + "q"].T, h @ w[p + "k"].T
-        v = k.reshape(T, G, d)                                       # the values are the keys as projected
+        v = k.reshape(T, G, d)                                       # the values: k straight out of its product
         q = unit_rms(q, self.eps) * w[p + "q.norm"]                  # over the whole projection, all heads at once
         k = unit_rms(k, self.eps) * w[p + "k.norm"]
         rot = m.get("rot")
