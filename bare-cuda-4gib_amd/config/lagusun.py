@@ -4,9 +4,9 @@ norms in groups; the embedding is multiplied by a constant; and a run of neighbo
 times with the same weights, each pass with a cache of its own, the stream being replaced before every pass (the first
 too) by a linear map of itself and the embedding's output plus a vector of the pass.
 
-``attention``    q and k only: a value head is its key head straight out of the product, untouched; q and k normed over their whole projection with a
-                 weight, then rotated (a head's first ``rot.dims`` elements, element i with i + dims/2); a row sees the keys of
-                 its own block of ``mask.size`` positions; softmax with a one in the denominator.
+``attention``    q and k only: a value head is its key head straight out of the product, untouched; q and k normed across
+                 all their heads together with a weight, then rotated (a head's first ``rot.dims`` elements in two halves); a
+                 row sees the keys of its own block of ``mask.size`` positions; softmax with a one in the denominator.
 ``attention_2``  q, k, v with biases; rotation with frequencies scaled by wavelength (``rot.scaling``); q and k divided by their
                  root mean square a head after the rotation, the values too; scores capped by ``softcap`` tanh(s / softcap); a
                  window of the last ``mask.size`` keys; the weight of a key is sigmoid(score + ``pb``[head]), no softmax.

@@ -26,7 +26,7 @@ int bc4g_embed_rows(const void* table, int table_dtype, const int32_t* ids, floa
 // x is the float residual stream; out has out_dtype; w has w_dtype.
 int bc4g_rmsnorm(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out,
                  int out_dtype, int n_rows, int hidden, float eps, void* stream);
-// The same with every row cut into `groups` equal consecutive parts, each divided by its own root mean square (w spans the row).
+// The same with every row in `groups` equal runs of neighbouring channels, each run brought to unit mean square by itself (w spans the row).
 int bc4g_rmsnorm_groups(const float* x, const int32_t* rows, const void* w, int w_dtype, void* out, int out_dtype, int n_rows,
                         int hidden, int groups, float eps, void* stream);
 // x = (keep ? x : 0) + scale * y + bias on the float32 stream x [n_rows, hidden] (y float32 of that shape; scale, bias float32

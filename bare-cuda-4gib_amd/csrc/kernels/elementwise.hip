@@ -33,7 +33,7 @@ __global__ void embed_gather_kernel(const TT* __restrict__ table, const int32_t*
 template <typename TW, typename TO>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
                                const TW* __restrict__ w, TO* __restrict__ out, int hidden, float eps, int groups) {
-  // (a workgroup is one of a row's `groups` equal consecutive parts, `hidden` elements each, normed by itself)
+  // (a workgroup is one of a row's `groups` equal runs of neighbouring channels, `hidden` elements each, normed by itself)
   __shared__ float scratch[16];
   const size_t row = blockIdx.x / groups, part = blockIdx.x % groups;
   const size_t src_row = rows ? static_cast<size_t>(rows[row]) : row;

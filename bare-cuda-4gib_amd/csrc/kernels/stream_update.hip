@@ -3,8 +3,8 @@
 //   update   x = (keep ? x : 0) + s * y + b      y a sublayer's float32 output, s and b one number a channel (each may be
 //            absent: 1 and 0), all element by element in float32; x is written back
 //   norm     and, if a weight is given, out = N(x) in the activations' dtype for whoever reads the stream next:
-//            the row cut into `groups` equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps),
-//            the whole times the weight
+//            the row in `groups` equal runs of neighbouring channels, a run r scaled by 1 / sqrt(mean(r^2) + eps) of its own,
+//            then every channel times its weight
 //   beside   out[t] = [x[t] | table[ids[t]] * factor] in the activations' dtype: the stream and the embedding of the
 //            same token side by side, the operand of a product over both
 //

@@ -167,8 +167,8 @@ def stream_update(x: torch.Tensor, y: torch.Tensor, scale: Optional[torch.Tensor
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None, groups: int = 1) -> torch.Tensor:
     """RMSNorm of rows of the float residual stream x [T, H]; with ``rows`` (int32
-    indices, the first n_rows are used) only those rows are normed.  ``groups``: a row is cut into that many equal
-    consecutive parts and each is divided by its own root mean square; the weight spans the row."""
+    indices, the first n_rows are used) only those rows are normed.  ``groups``: a row is that many equal runs of
+    neighbouring channels, each brought to unit mean square by itself; the weight spans the row."""
     _dev("rmsnorm", x, weight, rows)
     if x.dtype != torch.float32 or x.dim() != 2:
         raise KernelError(f"rmsnorm: x must be float32 [T, H], got {x.dtype} {tuple(x.shape)}")

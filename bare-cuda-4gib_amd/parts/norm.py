@@ -1,7 +1,7 @@
 """RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, with eps on the mean square and
 sum and rsqrt in float (reference: engine/kernels/rmsnorm.cu:16-41).  With ``offset`` the stored weight is
 counted from it: y = x * rsqrt(...) * (offset + w) -- a weight stored around zero has offset 1.  With ``groups`` the row
-is cut into that many equal consecutive parts and each is divided by its own root mean square; the weight spans the row."""
+is cut into that many equal runs of neighbouring channels, every run is brought to unit mean square by itself, and one weight spans the row."""
 from __future__ import annotations
 
 from typing import Dict

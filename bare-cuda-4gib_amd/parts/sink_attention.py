@@ -36,7 +36,7 @@ class SinkAttention(Part):
 
     bias        ``q.b``, ``k.b``, ``v.b`` are added to the projections
     values      "keys": there is no Wv -- a value head is its key head straight out of the product (what the keys go through afterwards does not touch it), vdim = dim
-    row_norm    q and k are normed over their whole projection, all heads at once, each with a weight that spans it
+    row_norm    q and k are normed across all their heads together (one mean square a token), each with a weight as wide as the row
                 (``q.norm`` [heads * dim], ``k.norm`` [kv_heads * dim]), before the rotation
     value_unit_norm  every value head divided by sqrt(mean(head^2) + eps), no weight; cached so
     block       instead of the window: a row sees the keys j <= p of its own block of ``block`` positions, counted from the

@@ -10,23 +10,23 @@ sequence's tokens from 0):
   embedding  x0 = E[token] * c                                 (c: ``embedding.scale``)
   layer      x += a1 * mixer(N1(x));  x += a2 * ff(N2(x))     (a1, a2: a vector each, element by element; a layer may
                                                                 have no ff)
-  N(v)       v cut into n equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps), the whole times g
+  N(v)       v cut into n equal runs of neighbouring channels; a run r becomes r / sqrt(mean(r^2) + eps); then all times g
   loop       layers a..b-1 run n times in a row with the same weights (each pass with a cache of its own); right before
              the first layer of pass t (t = 0 too)  x = W_in [x; x0] + s_t
   rotation   of a head's first ``dims`` elements, in two halves: (lo_i, hi_i) = (element i, element i + dims/2) turns by the
              angle t = p w_i at position p, w_i = base^(-2i/dims): lo' = lo cos t - hi sin t, hi' = hi cos t + lo sin t;
              with ``scaling`` the slow w_i are divided by a factor, the fast ones kept, those between blended
-  mixers     ``attention``    q = Wq h, k = Wk h, values = k straight out of its product; q and k each normed over the whole
-                              projection (all heads at once, with a weight), then rotated; a row sees the keys of its
+  mixers     ``attention``    q = Wq h, k = Wk h, values = k straight out of its product; q and k each normed across all
+                              heads together (one mean square a token, a weight a channel), then rotated; a row sees the keys of its
                               own block of ``mask.size`` positions up to itself; softmax with one more term, exp(0),
                               in the denominator
              ``attention_2``  q, k, v with biases; q and k rotated, then each head divided by its root mean square;
                               each value head divided by its root mean square; scores capped by c tanh(s / c); a row
-                              sees itself and the ``mask.size`` - 1 keys before it; the weight of a key is
-                              sigmoid(score + b_head), not normalised over keys
+                              sees itself and the ``mask.size`` - 1 keys before it; a key in sight counts with
+                              sigmoid(score + b_head), whatever the other keys score
   ff         sigmoid router over all experts, chosen by score + correction, the chosen scores divided by their sum and
-             multiplied by a constant; an expert is W_down gelu(W_up v) with the exact gelu; a shared expert of the same
-             form is added for every token
+             multiplied by a constant; an expert is W_down gelu(W_up v) with the exact gelu; one more expert of that form
+             stands outside the router and counts fully for every token
   output     logits = W_head N(x)
 """
 from __future__ import annotations
@@ -47,7 +47,7 @@ def unit_rms(v: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def grouped_norm(v: torch.Tensor, g: torch.Tensor, eps: float, groups: int) -> torch.Tensor:
-    """v [..., W] in ``groups`` consecutive parts, each divided by its own root mean square; the whole times g."""
+    """v [..., W] as ``groups`` runs of W / groups channels, every run through unit_rms by itself; then all channels times g."""
     parts = v.reshape(*v.shape[:-1], groups, v.shape[-1] // groups)
     return unit_rms(parts, eps).reshape(v.shape) * g
 
@@ -182,7 +182,7 @@ class PlainLagusun:
         H, G, d = m["heads"], m["kv_heads"], m["dim"]
         q, k = h @ w[p + "q"].T, h @ w[p + "k"].T
         v = k.reshape(T, G, d)                                       # the values: k straight out of its product
-        q = unit_rms(q, self.eps) * w[p + "q.norm"]                  # over the whole projection, all heads at once
+        q = unit_rms(q, self.eps) * w[p + "q.norm"]                  # one mean square over all heads of the token
         k = unit_rms(k, self.eps) * w[p + "k.norm"]
         rot = m.get("rot")
         freqs = scaled_frequencies(rot["dims"], rot["base"], rot.get("scaling")) if rot else torch.zeros(0, dtype=torch.float64)

@@ -276,7 +276,7 @@ def step_context(lengths, cached, slots):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("channels,groups", [(36, 3), (37, 1), (64, 4), (2500, 5), (4096, 2), (24, 24)])
 def test_norm_in_groups(dtype, channels, groups):
-    """Every part of a row divided by its own root mean square -- one part made a hundred times larger than the others
+    """Every run of a row brought to unit mean square by itself -- one run made a hundred times larger than the others
     leaves them as they are --, on all rows and on chosen ones."""
     from bare_cuda_4gib_amd.engine.spec import PartSpec
     from bare_cuda_4gib_amd.parts import build_part
